@@ -1,0 +1,131 @@
+/*
+ * pegainfer_kernels_blocks.h - building blocks of libpegainfer_kernels_hip.so that are not tied to one model family
+ * and exist in a bf16 and a true-fp32 instance: Dynamic-Tanh norms over an fp32 residual stream, squared-ReLU and
+ * SwiGLU activations, a strided / batched / grouped GEMM, attention over a paged LATENT cache (one compressed key/value
+ * vector plus one shared rotated key part per token), and sigmoid-scored grouped top-k expert routing.
+ *
+ * Conventions: device pointers; `dtype` 0 = bf16 bit patterns, 1 = float (storage of activations AND weights of that
+ * call); all arithmetic is fp32; stream last; every function only enqueues work and returns hipGetLastError() as int.
+ * Token-major activations ([rows, d], d contiguous).
+ */
+#ifndef PEGAINFER_KERNELS_BLOCKS_H
+#define PEGAINFER_KERNELS_BLOCKS_H
+
+#include <stdint.h>
+
+#include "pegainfer_kernels.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- residual stream in fp32 ---- */
+/* out[t, :] = embed[token_ids[t], :] widened to fp32 */
+pegainfer_status_t pegainfer_embed_f32(const void* embed, const uint32_t* token_ids, float* out, int32_t width,
+                                       int32_t n_tokens, int32_t dtype, pegainfer_stream_t stream);
+/* Dynamic Tanh: out = tanh(alpha * x) * w + b.  x fp32 [rows, d]; alpha a one-element tensor, w / b [d]; out [rows, d] */
+pegainfer_status_t pegainfer_dyt_norm(const float* x, const void* alpha, const void* w, const void* b, void* out,
+                                      int32_t d, int32_t rows, int32_t dtype, pegainfer_stream_t stream);
+/* x += dyt(y; post);  then, when next_w != NULL, out = dyt(x; next) - the post-norm of one sublayer, the residual sum and
+ * the pre-norm of the following sublayer in one pass over the row.  y, out [rows, d]; x fp32 [rows, d] in place */
+pegainfer_status_t pegainfer_dyt_add_norm(float* x, const void* y, const void* post_alpha, const void* post_w,
+                                          const void* post_b, const void* next_alpha, const void* next_w,
+                                          const void* next_b, void* out, int32_t d, int32_t rows, int32_t dtype,
+                                          pegainfer_stream_t stream);
+/* rows of an fp32 matrix gathered by index: out[i, :] = x[rows_index[i], :] (the positions whose logits are wanted) */
+pegainfer_status_t pegainfer_gather_rows_f32(const float* x, const int32_t* rows_index, float* out, int32_t d,
+                                             int32_t n_rows, pegainfer_stream_t stream);
+
+/* ---- activations ---- */
+/* out = max(x, 0)^2, elementwise (in place allowed) */
+pegainfer_status_t pegainfer_relu_sq(const void* x, void* out, int64_t n, int32_t dtype, pegainfer_stream_t stream);
+/* out[row, i] = silu(gu[row, i]) * gu[row, I + i]   (gate | up stacked along the row) */
+pegainfer_status_t pegainfer_silu_mul_rows(const void* gate_up, void* out, int32_t I, int32_t rows, int32_t dtype,
+                                           pegainfer_stream_t stream);
+
+/* ---- strided / batched / grouped GEMM:  y[row, g, m] = sum_k x[row, g, k] * w[g, m, k]  (+ epilogue) ----
+ * Dense form (tile_group == NULL): `rows` rows in each of `groups` groups.
+ * Grouped form: a device-side table of row tiles, each of <= 64 consecutive POSITIONS of a sorted list that belong to
+ * one group (expert); positions map to x / y rows through x_row_index / y_row_index (NULL = identity).  Tiles beyond
+ * *n_tiles exit; the grid is max_tiles wide.  The k order of every output is fixed, so a row's result does not depend
+ * on what else is in the launch. */
+enum { PEGAINFER_EPI_NONE = 0, PEGAINFER_EPI_RELU_SQ = 1, PEGAINFER_EPI_SIGMOID_GATE = 2 };
+typedef struct {
+  const void* x;
+  const void* w;
+  void* y;
+  int32_t x_dtype, w_dtype, y_dtype;
+  int32_t m, k, rows, groups;
+  int64_t x_row_stride, x_group_stride;
+  int64_t w_m_stride, w_k_stride, w_group_stride;
+  int64_t y_row_stride, y_group_stride;
+  const int32_t* tile_group;
+  const int32_t* tile_row0;
+  const int32_t* tile_rows;
+  const int32_t* n_tiles;
+  int32_t max_tiles;
+  const int32_t* x_row_index;
+  const int32_t* y_row_index;
+  int32_t epilogue;          /* SIGMOID_GATE: y *= sigmoid(gate[row * gate_row_stride + g]) */
+  const void* gate;
+  int32_t gate_dtype;
+  int64_t gate_row_stride;
+} pegainfer_gemm_desc;
+pegainfer_status_t pegainfer_gemm_strided(const pegainfer_gemm_desc* d, pegainfer_stream_t stream);
+
+/* ---- attention over a paged latent cache ----
+ * Cache: page-first; one layer's entry of one token = [c: rank values | kr: rot values], at
+ *   cache + page * page_stride + layer_off + slot * (rank + rot)        (elements of `dtype`).
+ * A step's token rows carry their request (token_req), their position in that request (positions) and the request's
+ * page list (page_ids[page_indptr[req] ...]).
+ *
+ * pegainfer_latent_prep: per token row, from one projection row  [ q: heads * (nope + rot) | ... | dkv: rank + rot ]:
+ *   c  = dkv[:rank] / sqrt(mean(dkv[:rank]^2) + eps) * c_norm_w            -> cache entry [0, rank)
+ *   kr = rotate_half(dkv[rank:], position)                                   -> cache entry [rank, rank + rot)
+ *   qc[t, h, rank:] = rotate_half(q[t, h, nope:], position)   (fp32; qc[t, h, :rank] is filled by the absorb GEMM)
+ * rotate_half acts on the first rot_dims of the rot values: pair (i, i + rot_dims / 2), angle position * inv_freq[i],
+ * both in fp32; the remaining values pass through. */
+pegainfer_status_t pegainfer_latent_prep(const void* proj, int64_t proj_row_stride, int64_t dkv_offset,
+                                         const void* c_norm_w, float eps, const float* inv_freq, int32_t rot_dims,
+                                         const int32_t* positions, const int32_t* token_req, const int32_t* page_indptr,
+                                         const int32_t* page_ids, void* cache, int64_t page_stride, int64_t layer_off,
+                                         int32_t page_size, float* qc, int32_t heads, int32_t nope, int32_t rot,
+                                         int32_t rank, int32_t n_tokens, int32_t dtype, pegainfer_stream_t stream);
+/* Causal softmax attention of every (token, head) row over its request's cache entries 0 .. position:
+ *   score_j = (qc[t, h, :] . entry_j) * scale;  o_lat[t, h, :] = sum_j softmax(score)_j * entry_j[:rank]
+ * qc fp32 [T, heads, rank + rot], o_lat fp32 [T, heads, rank]; scores, weights and sums in fp32.
+ * workspace: fp32 scratch of pegainfer_latent_attention_workspace(...) floats (NULL allowed when that is 0). */
+int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, int32_t rank, int32_t max_kv_len);
+pegainfer_status_t pegainfer_latent_attention(const float* qc, float* o_lat, const void* cache, int64_t page_stride,
+                                              int64_t layer_off, int32_t page_size, const int32_t* positions,
+                                              const int32_t* token_req, const int32_t* page_indptr,
+                                              const int32_t* page_ids, int32_t heads, int32_t rank, int32_t rot,
+                                              float scale, int32_t n_tokens, int32_t max_kv_len, float* workspace,
+                                              int32_t dtype, pegainfer_stream_t stream);
+
+/* ---- routed experts ----
+ * Router: z = W_r h (fp32 accumulation of the stored values), s = sigmoid(z), choice = s + correction (NULL = none).
+ * The experts form n_groups equal groups of neighbours; a group's score is the sum of its two largest choices (of its
+ * one choice when a group is a single expert); only the keep_groups best groups stay eligible; the `top` largest
+ * eligible choices are taken (ties: the lower index).  out_expert / out_weight [rows, top]; the weight is s of the
+ * chosen expert, not renormalised. */
+pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_router, const void* correction,
+                                                   int32_t* out_expert, float* out_weight, int32_t d, int32_t experts,
+                                                   int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                                   int32_t dtype, pegainfer_stream_t stream);
+/* Sort the rows * top (row, choice) pairs by expert into a position list and cut it into row tiles of <= 64 positions:
+ *   pos_pair[p] = pair index (row * top + choice) at position p;  pos_row[p] = its row
+ *   tile_group / tile_row0 / tile_rows [max_tiles], *n_tiles;  max_tiles >= ceil(pairs / 64) + experts
+ * One workgroup, counters in LDS (experts <= 8192).  The order inside an expert is arbitrary; results do not depend on it. */
+pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, int32_t top, int32_t experts,
+                                        int32_t* pos_pair, int32_t* pos_row, int32_t* tile_group, int32_t* tile_row0,
+                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles,
+                                        pegainfer_stream_t stream);
+/* out[row, :] = sum_c weight[row, c] * y_pairs[row * top + c, :]   (c ascending; y_pairs fp32) */
+pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,
+                                           int32_t rows, int32_t dtype, pegainfer_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PEGAINFER_KERNELS_BLOCKS_H */

@@ -97,6 +97,10 @@ pegainfer_sched_t pegainfer_sched_create_qwen3(void* model, uint64_t seed, const
  * decode per iteration; sampled requests draw through pegainfer_qwen35_sample, logprobs through pegainfer_qwen35_logprobs
  * (round 4; echo logits are not computed for this model).  `model` is a pegainfer_qwen35_t. */
 pegainfer_sched_t pegainfer_sched_create_qwen35(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop);
+/* scheduler over the Duguzen runtime (pegainfer_duguzen.h): every plan - Prefill, Decode, Unified - is ONE call of
+ * pegainfer_duguzen_step over all of the iteration's requests; sampled requests draw through pegainfer_duguzen_sample,
+ * logprobs through pegainfer_duguzen_logprobs (no prompt echo).  `model` is a pegainfer_duguzen_t. */
+pegainfer_sched_t pegainfer_sched_create_duguzen(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop);
 void pegainfer_sched_destroy(pegainfer_sched_t s);
 
 /* EngineHandle::submit: returns the RequestId the events carry (ids count up from 0 in submission order) */

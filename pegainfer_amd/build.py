@@ -51,8 +51,9 @@ def _run(cmd):
 def _compile(src, extra, headers, objdir=None):
     obj = os.path.join(objdir or OBJDIR, os.path.basename(src) + ".o")
     if _newer([src] + headers, obj):
+        # no packed-fp32 VALU forms (v_pk_*_f32): hipcc -O3 otherwise forms them from plain float code
         _run([_hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall",
-              "-Wno-unused-function", "-I", os.path.join(ROOT, "include"), "-I", CSRC] + extra +
+              "-Wno-unused-function", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", os.path.join(ROOT, "include"), "-I", CSRC] + extra +
              ["-c", src, "-o", obj])
     return obj
 

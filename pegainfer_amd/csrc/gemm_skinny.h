@@ -788,10 +788,12 @@ inline bool skinny_is_resident(int nw, int T, int K) {
   const int nb = T <= 16 ? 1 : T <= 32 ? 2 : 4;
   return (long)T * K * 2 <= kSkinnyResidentBytes && (long)T * K * 2 + 8 * nw * nb * 64 * 16 + 256 <= 160 * 1024;
 }
-// 2 <= T <= 64, K % 64 == 0
+// 2 <= T <= 64, K % 64 == 0; above 8 token rows K % 128 == 0 as well: the staged x rows are swizzled by XOR-ing the
+// 16-byte chunk index with (t & 15), which stays inside the row only when the row has a multiple of 16 chunks
+// (rows 0..7 flip the low three bits only, and K % 64 == 0 already makes the chunk count a multiple of 8)
 template <int EPI>
 inline bool skinny_dispatch(const GemvFusedArgs& a, hipStream_t s) {
-  if (a.T < 2 || a.T > 64 || (a.K & 63) != 0) return false;
+  if (a.T < 2 || a.T > 64 || (a.K & 63) != 0 || (a.T > 8 && (a.K & 127) != 0)) return false;
   constexpr int NW = EPI == kEpiSilu ? 2 : 1;
   const bool resident = skinny_is_resident(NW, a.T, a.K);
   if (a.T <= 16) { if (resident) skinny_launch_resident<1, EPI>(a, s); else skinny_launch<1, EPI>(a, s); }

@@ -11,6 +11,7 @@
 
 #include "pegainfer_qwen3.h"
 #include "pegainfer_qwen35.h"
+#include "pegainfer_duguzen.h"
 #include "pegainfer_scheduler.h"
 
 namespace psched {
@@ -274,10 +275,75 @@ struct Qwen35Exec {
   }
 };
 
+// Executor over the Duguzen runtime (pegainfer_duguzen.h).  Its step function takes prompts and single tokens of several
+// requests as ONE batch, so a Prefill, a Decode and a Unified plan are all the same call; sampled requests draw from their
+// wanted row afterwards, logprobs read the row's fp32 logits.
+struct DuguzenExec {
+  pegainfer_duguzen_t model;
+  std::unordered_set<uint32_t> stop;
+  std::unordered_map<uint64_t, int32_t> slot;
+  std::string err;
+  static DuguzenExec* E(void* u) { return (DuguzenExec*)u; }
+  static int32_t page_size(void* u) { return pegainfer_duguzen_page_size(E(u)->model); }
+  static int32_t max_request_pages(void* u) { return pegainfer_duguzen_capacity_pages(E(u)->model); }
+  static int32_t available_pages(void* u) { return pegainfer_duguzen_available_pages(E(u)->model); }
+  static int32_t max_batch_size(void* u) { return pegainfer_duguzen_max_batch_size(E(u)->model); }
+  static int32_t is_stop_token(void* u, uint32_t t) { return E(u)->stop.count(t) ? 1 : 0; }
+  static int32_t drop_request(void* u, uint64_t id) {
+    auto* e = E(u);
+    auto it = e->slot.find(id);
+    if (it == e->slot.end()) return 0;
+    const int32_t rc = pegainfer_duguzen_drop_request(e->model, it->second);
+    e->slot.erase(it);
+    return rc;
+  }
+  static const char* last_error(void* u) { return E(u)->err.c_str(); }
+  static bool greedy(float t, int32_t k, float p) { return (t <= 0.0f || k == 1) && p >= 1.0f; }
+  static int32_t execute(void* u, int32_t n_pf, int32_t n_dec, const uint64_t* ids, const int32_t* lens,
+                         const uint32_t* tokens, const float* temp, const int32_t* top_k, const float* top_p,
+                         const float* rv, uint32_t* out) {
+    auto* e = E(u);
+    auto fail = [&](const char* what) {
+      const char* m = pegainfer_duguzen_last_error(e->model);
+      e->err = std::string(what) + ": " + (m ? m : "");
+      return -1;
+    };
+    const int n = n_pf + n_dec;
+    std::vector<int32_t> slots(n), toks(n);
+    for (int i = 0; i < n; ++i) {
+      if (i < n_pf) {
+        const int32_t r = pegainfer_duguzen_new_request(e->model);
+        if (r < 0) return fail("new_request");
+        e->slot[ids[i]] = r;
+        slots[i] = r;
+      } else {
+        auto it = e->slot.find(ids[i]);
+        if (it == e->slot.end()) { e->err = "decode request without model state"; return -1; }
+        slots[i] = it->second;
+      }
+    }
+    if (pegainfer_duguzen_step(e->model, n, slots.data(), lens, tokens, -1, nullptr, nullptr, toks.data())) return fail("step");
+    for (int i = 0; i < n; ++i) {
+      if (!greedy(temp[i], top_k[i], top_p[i]) &&
+          pegainfer_duguzen_sample(e->model, i, temp[i], top_k[i], top_p[i], rv[i], &toks[i]))
+        return fail("sample");
+      out[i] = (uint32_t)toks[i];
+    }
+    return 0;
+  }
+  static int32_t logprobs(void* u, int32_t row, uint32_t token, int32_t top_k, float* lp, uint32_t* ids, float* vals) {
+    auto* e = E(u);
+    const int32_t rc = pegainfer_duguzen_logprobs(e->model, row, token, top_k, lp, ids, vals);
+    if (rc < 0) { const char* m = pegainfer_duguzen_last_error(e->model); e->err = m ? m : "logprobs failed"; }
+    return rc;
+  }
+};
+
 struct Scheduler {
   pegainfer_executor_vtbl ex;
   Qwen3Exec* owned = nullptr;
   Qwen35Exec* owned35 = nullptr;
+  DuguzenExec* owned_dz = nullptr;
   Rng rng;
   std::vector<Active> active;
   std::vector<Pending> deferred;
@@ -534,10 +600,24 @@ pegainfer_sched_t pegainfer_sched_create_qwen35(void* model, uint64_t seed, cons
   s->owned35 = e;
   return s;
 }
+pegainfer_sched_t pegainfer_sched_create_duguzen(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop) {
+  if (!model) return nullptr;
+  auto* e = new psched::DuguzenExec();
+  e->model = model;
+  for (int i = 0; i < n_stop; ++i) e->stop.insert(stop_tokens[i]);
+  pegainfer_executor_vtbl v{sizeof(pegainfer_executor_vtbl), e, &psched::DuguzenExec::page_size, &psched::DuguzenExec::max_request_pages,
+                            &psched::DuguzenExec::available_pages, &psched::DuguzenExec::is_stop_token,
+                            &psched::DuguzenExec::drop_request, &psched::DuguzenExec::execute, &psched::DuguzenExec::last_error,
+                            &psched::DuguzenExec::max_batch_size, &psched::DuguzenExec::logprobs, nullptr, nullptr};
+  Scheduler* s = static_cast<Scheduler*>(pegainfer_sched_create(&v, seed));
+  s->owned_dz = e;
+  return s;
+}
 void pegainfer_sched_destroy(pegainfer_sched_t s) {
   if (!s) return;
   delete SC(s)->owned;
   delete SC(s)->owned35;
+  delete SC(s)->owned_dz;
   delete SC(s);
 }
 uint64_t pegainfer_sched_submit_ex(pegainfer_sched_t s, const uint32_t* prompt_tokens, int32_t n_tokens, int32_t max_tokens,

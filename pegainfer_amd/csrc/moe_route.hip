@@ -1,0 +1,169 @@
+// Routed feed-forward: the router and the bookkeeping around the expert GEMMs (which run on the grouped form of
+// pegainfer_gemm_strided).
+//   route_kernel    one workgroup per token row: fp32 router logits (a wave per expert, lanes over the width), sigmoid
+//                   scores, the correction added for the CHOICE only, group scores = the two largest choices of a group,
+//                   the best `keep` groups stay eligible, then the `top` largest eligible choices; weights = the plain
+//                   sigmoid scores of the chosen experts.  Selection is serial in one thread: E is tens to hundreds, and
+//                   ties go to the lower index.
+//   sort_kernel     (row, choice) pairs bucketed by expert with LDS counters, an exclusive scan, and the table of <= 64-row
+//                   tiles the grouped GEMM walks.  The order of pairs inside an expert comes from atomics; every pair owns
+//                   its output row, so results do not depend on it.
+//   combine_kernel  out[row] = sum over the row's choices, in choice order, of weight * expert output (fp32 sum).
+#include "common.h"
+#include "typed.h"
+#include "pegainfer_kernels_blocks.h"
+
+namespace pk {
+
+template <typename A>
+__global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, const A* __restrict__ wr,
+                                                    const A* __restrict__ corr, int32_t* __restrict__ out_e,
+                                                    float* __restrict__ out_w, int d, int E, int G, int keep, int top) {
+  extern __shared__ float sm[];
+  float* s = sm;            // [E] sigmoid scores
+  float* ch = sm + E;       // [E] choice scores (eligible) or -inf
+  float* gs = sm + 2 * E;   // [G] group scores
+  const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const A* x = h + (size_t)row * d;
+  for (int e = wave; e < E; e += 4) {
+    const A* w = wr + (size_t)e * d;
+    float a = 0.f;
+    for (int i = lane; i < d; i += 64) a = fmaf(ld(x + i), ld(w + i), a);
+    a = wave_sum(a);
+    if (lane == 0) {
+      const float sc = sigmoid_f(a);
+      s[e] = sc;
+      ch[e] = corr ? sc + ld(corr + e) : sc;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  if (G > 1) {
+    const int per = E / G;
+    for (int g = 0; g < G; ++g) {
+      float b0 = -INFINITY, b1 = -INFINITY;
+      for (int i = 0; i < per; ++i) {
+        const float v = ch[g * per + i];
+        if (v > b0) { b1 = b0; b0 = v; } else if (v > b1) b1 = v;
+      }
+      gs[g] = per >= 2 ? b0 + b1 : b0;
+    }
+    // drop the G - keep worst groups: repeatedly take the best remaining group, mark it kept (score := NaN-free flag)
+    for (int k = 0; k < keep; ++k) {
+      int best = -1;
+      for (int g = 0; g < G; ++g)
+        if (gs[g] != INFINITY && (best < 0 || gs[g] > gs[best])) best = g;
+      if (best >= 0) gs[best] = INFINITY;   // kept
+    }
+    for (int g = 0; g < G; ++g)
+      if (gs[g] != INFINITY)
+        for (int i = 0; i < per; ++i) ch[g * per + i] = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    int best = 0;
+    float bv = -INFINITY;
+    bool found = false;
+    for (int e = 0; e < E; ++e) {
+      const float v = ch[e];
+      if (v == -INFINITY) continue;         // taken or not eligible
+      if (!found || v > bv) { best = e; bv = v; found = true; }
+    }
+    out_e[(size_t)row * top + k] = best;
+    out_w[(size_t)row * top + k] = found ? s[best] : 0.f;
+    if (found) ch[best] = -INFINITY;
+  }
+}
+
+__global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restrict__ expert, int n_pairs, int top, int E,
+                                                         int32_t* __restrict__ pos_pair, int32_t* __restrict__ pos_row,
+                                                         int32_t* __restrict__ tile_group, int32_t* __restrict__ tile_row0,
+                                                         int32_t* __restrict__ tile_rows, int32_t* __restrict__ n_tiles,
+                                                         int max_tiles) {
+  extern __shared__ int cnt[];   // [E] counts, then [E] cursors
+  int* cur = cnt + E;
+  for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += 256) atomicAdd(&cnt[expert[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int off = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cnt[e];
+      cur[e] = off;
+      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += 64, ++nt) {
+        tile_group[nt] = e;
+        tile_row0[nt] = off + r0;
+        tile_rows[nt] = min(64, c - r0);
+      }
+      off += c;
+    }
+    *n_tiles = nt;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += 256) {
+    const int at = atomicAdd(&cur[expert[p]], 1);
+    pos_pair[at] = p;
+    pos_row[at] = p / top;
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                            A* __restrict__ out, int d, int top) {
+  const int row = blockIdx.x;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    float a = 0.f;
+    for (int c = 0; c < top; ++c) a = fmaf(w[(size_t)row * top + c], y[((size_t)row * top + c) * d + i], a);
+    st(out + (size_t)row * d + i, a);
+  }
+}
+
+}  // namespace pk
+
+extern "C" {
+using namespace pk;
+
+pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_router, const void* correction,
+                                                   int32_t* out_expert, float* out_weight, int32_t d, int32_t experts,
+                                                   int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                                   int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0) return 0;
+  if (n_groups < 1) n_groups = 1;
+  if (experts <= 0 || experts % n_groups || top <= 0 || top > experts || keep_groups < 1 || keep_groups > n_groups ||
+      (size_t)(2 * experts + n_groups) * 4 > 60000)
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  const size_t smem = (size_t)(2 * experts + n_groups) * sizeof(float);
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        route_kernel<A><<<rows, 256, smem, as_stream(stream)>>>(static_cast<const A*>(h), static_cast<const A*>(w_router),
+                                                                static_cast<const A*>(correction), out_expert, out_weight, d,
+                                                                experts, n_groups, keep_groups, top);
+      }))
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, int32_t top, int32_t experts,
+                                        int32_t* pos_pair, int32_t* pos_row, int32_t* tile_group, int32_t* tile_row0,
+                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles,
+                                        pegainfer_stream_t stream) {
+  if (n_pairs <= 0) return 0;
+  if (experts <= 0 || experts > 7000 || max_tiles < (n_pairs + 63) / 64 + experts)
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  route_sort_kernel<<<1, 256, (size_t)2 * experts * sizeof(int), as_stream(stream)>>>(
+      expert, n_pairs, top, experts, pos_pair, pos_row, tile_group, tile_row0, tile_rows, n_tiles, max_tiles);
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,
+                                           int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0) return 0;
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        route_combine_kernel<A><<<rows, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<A*>(out), d, top);
+      }))
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+}  // extern "C"

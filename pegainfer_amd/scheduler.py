@@ -57,8 +57,8 @@ class Scheduler:
     def over_engine(cls, engine, seed=42, stop_tokens=()):
         lib = ffi.host_lib()
         st = np.ascontiguousarray(list(stop_tokens), dtype=np.uint32)
-        create = lib.pegainfer_sched_create_qwen35 if type(engine).__name__ == "Qwen35Engine" \
-            else lib.pegainfer_sched_create_qwen3
+        create = {"Qwen35Engine": lib.pegainfer_sched_create_qwen35,
+                  "DuguzenEngine": lib.pegainfer_sched_create_duguzen}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
         h = create(engine.h, seed, st.ctypes.data if st.size else None, int(st.size))
         return cls(h, keep=engine)
 
