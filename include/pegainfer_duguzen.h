@@ -83,9 +83,10 @@ int32_t pegainfer_duguzen_debug_hidden(pegainfer_duguzen_t m, int32_t layer_run,
 /* device time of the last step (hipEvent pair on the model stream), ms; bytes of weights on the device */
 float pegainfer_duguzen_last_step_ms(pegainfer_duguzen_t m);
 int64_t pegainfer_duguzen_weight_bytes(pegainfer_duguzen_t m);
-/* 0 (default): dense projections of a bf16 model run on the library's tuned GEMM routes (gemm_cuda); 1: everything on the
- * strided fp32-accumulating tile kernel (the form the fp32 model always uses) - the two agree to bf16 rounding */
-int32_t pegainfer_duguzen_set_plain_gemm(pegainfer_duguzen_t m, int32_t on);
+/* 0 (default): a bf16 model runs its dense projections on the library's tuned GEMM routes (gemm_cuda) and its attention
+ * on the matrix-core form; 1: everything on the plain fp32-arithmetic kernels (the forms the fp32 model always uses) - the
+ * two agree to bf16 rounding */
+int32_t pegainfer_duguzen_set_plain_kernels(pegainfer_duguzen_t m, int32_t on);
 
 #ifdef __cplusplus
 }

@@ -93,15 +93,23 @@ pegainfer_status_t pegainfer_latent_prep(const void* proj, int64_t proj_row_stri
                                          int32_t rank, int32_t n_tokens, int32_t dtype, pegainfer_stream_t stream);
 /* Causal softmax attention of every (token, head) row over its request's cache entries 0 .. position:
  *   score_j = (qc[t, h, :] . entry_j) * scale;  o_lat[t, h, :] = sum_j softmax(score)_j * entry_j[:rank]
- * qc fp32 [T, heads, rank + rot], o_lat fp32 [T, heads, rank]; scores, weights and sums in fp32.
- * workspace: fp32 scratch of pegainfer_latent_attention_workspace(...) floats (NULL allowed when that is 0). */
-int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, int32_t rank, int32_t max_kv_len);
+ * qc fp32 [T, heads, rank + rot], o_lat fp32 [T, heads, rank]; scores, running maxima / sums and accumulators in fp32.
+ * A row's keys are cut into splits of split_keys (<= 0: 1024) that run in parallel and are merged in split order;
+ * workspace: fp32 scratch of pegainfer_latent_attention_workspace(...) floats (NULL allowed when that is 0).
+ * Two forms.  tile_row0 == NULL: the plain form, any sizes, bf16 or fp32 cache, fp32 arithmetic throughout.
+ * tile_row0 != NULL: the matrix-core form for a bf16 cache (pegainfer_latent_attention_tiled_ok says whether the sizes fit):
+ * the flattened rows t * heads + h are cut by the caller into n_tiles runs of <= 64 rows that stay inside one request
+ * (tile_row0[i], tile_rows[i]); q and the softmax weights are rounded to bf16 where they enter the matrix cores. */
+int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, int32_t rank, int32_t max_kv_len,
+                                             int32_t split_keys);
+int32_t pegainfer_latent_attention_tiled_ok(int32_t rank, int32_t rot, int64_t page_stride, int64_t layer_off, int32_t dtype);
 pegainfer_status_t pegainfer_latent_attention(const float* qc, float* o_lat, const void* cache, int64_t page_stride,
                                               int64_t layer_off, int32_t page_size, const int32_t* positions,
                                               const int32_t* token_req, const int32_t* page_indptr,
                                               const int32_t* page_ids, int32_t heads, int32_t rank, int32_t rot,
-                                              float scale, int32_t n_tokens, int32_t max_kv_len, float* workspace,
-                                              int32_t dtype, pegainfer_stream_t stream);
+                                              float scale, int32_t n_tokens, int32_t max_kv_len, int32_t split_keys,
+                                              float* workspace, const int32_t* tile_row0, const int32_t* tile_rows,
+                                              int32_t n_tiles, int32_t dtype, pegainfer_stream_t stream);
 
 /* ---- routed experts ----
  * Router: z = W_r h (fp32 accumulation of the stored values), s = sigmoid(z), choice = s + correction (NULL = none).

@@ -25,7 +25,7 @@ namespace pk {
 
 constexpr int kLatKeys = 256;        // keys per round = threads per workgroup
 constexpr int kLatAcc = 4;           // latent dims per thread: rank <= 1024
-constexpr int kLatSplitKeys = 1024;  // keys per split of a row
+constexpr int kLatSplitKeys = 1024;  // default keys per split of a row
 
 __device__ __forceinline__ float block_max256(float v, float* red) {
   v = wave_max(v);
@@ -96,15 +96,15 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
                                                           const int32_t* __restrict__ token_req,
                                                           const int32_t* __restrict__ page_indptr,
                                                           const int32_t* __restrict__ page_ids, int H, int r, int dr,
-                                                          float scale, float* __restrict__ partial, int max_splits) {
+                                                          float scale, float* __restrict__ partial, int max_splits, int split_keys) {
   extern __shared__ float smem[];
   __shared__ float red[4];
   const int t = blockIdx.x, h = blockIdx.y, split = blockIdx.z, tid = threadIdx.x;
   const int E = r + dr;
   const int n_keys = positions[t] + 1;
-  const int n_splits = (n_keys + kLatSplitKeys - 1) / kLatSplitKeys;
+  const int n_splits = (n_keys + split_keys - 1) / split_keys;
   if (split >= n_splits) return;
-  const int j_lo = split * kLatSplitKeys, j_hi = min(n_keys, j_lo + kLatSplitKeys);
+  const int j_lo = split * split_keys, j_hi = min(n_keys, j_lo + split_keys);
   float* q = smem;            // [E]
   float* p = smem + E;        // [kLatKeys]
   const float* qrow = qc + ((int64_t)t * H + h) * E;
@@ -159,9 +159,9 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
 
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(float* __restrict__ o_lat, const float* __restrict__ partial,
                                                                 const int32_t* __restrict__ positions, int H, int r,
-                                                                int max_splits) {
+                                                                int max_splits, int split_keys) {
   const int t = blockIdx.x, h = blockIdx.y;
-  const int n_splits = (positions[t] + 1 + kLatSplitKeys - 1) / kLatSplitKeys;
+  const int n_splits = (positions[t] + split_keys) / split_keys;
   if (n_splits <= 1) return;
   const float* part = partial + ((int64_t)t * H + h) * max_splits * (r + 2);
   float m = -INFINITY;
@@ -175,7 +175,161 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(float* __restric
   }
 }
 
-static inline int latent_max_splits(int max_kv_len) { return std::max(1, (max_kv_len + kLatSplitKeys - 1) / kLatSplitKeys); }
+// ------------------------------------------------------------------ MFMA form (bf16 cache)
+// One workgroup = 64 consecutive (token, head) rows of ONE request (4 waves x 16 rows) against key tiles of 32 cache entries,
+// v_mfma_f32_16x16x32_bf16 for both products:
+//   scores^T [32 keys x 16 rows]  = entries [32 x E] . q^T          A = entry rows from LDS, B = the wave's q rows (bf16 in LDS)
+//   out^T    [16 dims x 16 rows] += c^T [16 x 32 keys] . p^T        A = the latent tile TRANSPOSED in LDS, B = the lane's own p
+// The score MFMA leaves lane (row l15, group g) with the scores of keys 4g..4g+3 and 16+4g..16+4g+3 of its row - exactly the
+// eight values the second product wants from that lane as its B operand, provided the reduction index is numbered
+// kidx = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4); the transposed latent tile is written in that numbering, so the
+// weights never move between lanes.  Every head of a token reads the same entries, so a tile of 64 rows (8 tokens x 8 heads,
+// or one decoded token's heads) shares each staged key tile.  Softmax state (max, sum) and the output accumulators are fp32;
+// q and the weights are rounded to bf16 where they enter the matrix cores.  Keys are split over blockIdx.y like the plain form.
+constexpr int kTileRows = 64, kTileKeys = 32;
+
+template <int ND>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __restrict__ qc, float* __restrict__ o_lat,
+                                                               const uint16_t* __restrict__ cache, int64_t page_stride,
+                                                               int64_t layer_off, int page_size,
+                                                               const int32_t* __restrict__ positions,
+                                                               const int32_t* __restrict__ token_req,
+                                                               const int32_t* __restrict__ page_indptr,
+                                                               const int32_t* __restrict__ page_ids,
+                                                               const int32_t* __restrict__ tile_row0,
+                                                               const int32_t* __restrict__ tile_rows, int H, int r, int dr,
+                                                               float scale, float* __restrict__ partial, int max_splits,
+                                                               int split_keys) {
+  extern __shared__ __align__(16) uint8_t lat_smem[];
+  const int E = r + dr, Epad = (E + 31) & ~31;
+  const int qs = Epad + 8, cs = Epad + 8, ts = kTileKeys + 8;      // LDS row strides (bf16 elements), 16-byte multiples
+  uint16_t* Qs = reinterpret_cast<uint16_t*>(lat_smem);            // [64][qs]
+  uint16_t* Ck = Qs + kTileRows * qs;                              // [32][cs]
+  uint16_t* Ct = Ck + kTileKeys * cs;                              // [ND * 16][ts]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l15 = lane & 15, g = lane >> 4;
+  const int row0 = tile_row0[blockIdx.x], cnt = tile_rows[blockIdx.x], split = blockIdx.y;
+  const int t_first = row0 / H, t_last = (row0 + cnt - 1) / H;
+  const int pmax = positions[t_last];
+  const int j_lo = split * split_keys;
+  if (j_lo > pmax) return;
+  const int j_hi = min(pmax + 1, j_lo + split_keys);
+  const int32_t* pages = page_ids + page_indptr[token_req[t_first]];
+  for (int i = tid; i < kTileRows * Epad; i += 256) {
+    const int row = i / Epad, k = i - row * Epad;
+    Qs[row * qs + k] = (row < cnt && k < E) ? f2bf(qc[(int64_t)(row0 + row) * E + k]) : (uint16_t)0;
+  }
+  for (int i = tid; i < kTileKeys * (Epad - E); i += 256) Ck[(i / (Epad - E)) * cs + E + i % (Epad - E)] = 0;
+  for (int i = tid; i < (ND * 16 - r) * kTileKeys; i += 256) Ct[(r + i / kTileKeys) * ts + i % kTileKeys] = 0;
+  const int my_row = wave * 16 + l15;
+  const int pq = my_row < cnt ? positions[(row0 + my_row) / H] : -1;
+  f32x4 o[ND];
+#pragma unroll
+  for (int d = 0; d < ND; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int nchunk = E >> 3;
+  for (int j0 = j_lo; j0 < j_hi; j0 += kTileKeys) {
+    __syncthreads();
+    for (int c = tid; c < kTileKeys * nchunk; c += 256) {
+      const int kk = c / nchunk, ch = c - kk * nchunk;
+      const int j = min(j0 + kk, j_hi - 1);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(latent_entry(cache, page_stride, layer_off, page_size, pages, j, E) + ch * 8);
+      *reinterpret_cast<u32x4*>(Ck + kk * cs + ch * 8) = v;
+      if (ch * 8 < r) {
+        const int kidx = kk < 16 ? 8 * (kk >> 2) + (kk & 3) : 8 * ((kk - 16) >> 2) + 4 + (kk & 3);
+        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int d = ch * 8 + i;
+          if (d < r) Ct[d * ts + kidx] = (uint16_t)(i & 1 ? wv[i >> 1] >> 16 : wv[i >> 1] & 0xFFFFu);
+        }
+      }
+    }
+    __syncthreads();
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < Epad; kb += 32) {
+      const bf16x8_t qv = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Qs + my_row * qs + kb + g * 8));
+      const bf16x8_t k0 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ck + l15 * cs + kb + g * 8));
+      const bf16x8_t k1 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ck + (16 + l15) * cs + kb + g * 8));
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qv, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qv, s1, 0, 0, 0);
+    }
+    float sc[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = j0 + (i < 4 ? 4 * g + i : 16 + 4 * g + i - 4);
+      const float v = (i < 4 ? s0[i] : s1[i - 4]) * scale;
+      sc[i] = (j <= pq && j < j_hi) ? v : -INFINITY;
+      mx = fmaxf(mx, sc[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = expf(m - m_use);
+    float ps[8], lsum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      ps[i] = bf16_round_f(expf(sc[i] - m_use));     // the sum uses the weights as the matrix core sees them
+      lsum += ps[i];
+    }
+    lsum += __shfl_xor(lsum, 16, kWave);
+    lsum += __shfl_xor(lsum, 32, kWave);
+    l = l * corr + lsum;
+    m = m_new;
+    const u32x4 pw = {pack_bf2(ps[0], ps[1]), pack_bf2(ps[2], ps[3]), pack_bf2(ps[4], ps[5]), pack_bf2(ps[6], ps[7])};
+    const bf16x8_t pv = __builtin_bit_cast(bf16x8_t, pw);
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      if (d * 16 >= r) break;
+      o[d] *= corr;
+      const bf16x8_t cv = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ct + (d * 16 + l15) * ts + g * 8));
+      o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cv, pv, o[d], 0, 0, 0);
+    }
+  }
+  if (my_row >= cnt) return;
+  const int own_splits = (pq + split_keys) / split_keys;
+  const int64_t grow = row0 + my_row;
+  if (own_splits == 1) {
+    if (split != 0) return;
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      const int dd = d * 16 + 4 * g;
+      if (dd < r) *reinterpret_cast<f32x4*>(o_lat + grow * r + dd) = o[d] * inv;
+    }
+  } else if (split < own_splits) {
+    float* part = partial + (grow * max_splits + split) * (r + 2);
+    if (g == 0) { part[0] = m; part[1] = l; }
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      const int dd = d * 16 + 4 * g;
+      if (dd < r) { part[2 + dd] = o[d][0]; part[3 + dd] = o[d][1]; part[4 + dd] = o[d][2]; part[5 + dd] = o[d][3]; }
+    }
+  }
+}
+
+template <int ND>
+static void latent_attn_mfma_launch(const float* qc, float* o_lat, const uint16_t* cache, int64_t page_stride, int64_t layer_off,
+                                    int page_size, const int32_t* positions, const int32_t* token_req,
+                                    const int32_t* page_indptr, const int32_t* page_ids, const int32_t* tile_row0,
+                                    const int32_t* tile_rows, int n_tiles, int H, int r, int dr, float scale, float* ws, int sp,
+                                    int split_keys, hipStream_t s) {
+  const int Epad = (r + dr + 31) & ~31;
+  const int lds = ((kTileRows + kTileKeys) * (Epad + 8) + ND * 16 * (kTileKeys + 8)) * 2;
+  auto kern = &latent_attn_mfma_kernel<ND>;
+  static const bool once = (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                160 * 1024), true);
+  (void)once;
+  kern<<<dim3(n_tiles, sp), 256, lds, s>>>(qc, o_lat, cache, page_stride, layer_off, page_size, positions, token_req, page_indptr,
+                                           page_ids, tile_row0, tile_rows, H, r, dr, scale, ws, sp, split_keys);
+}
+
+static inline int latent_split_keys(int split_keys) { return split_keys > 0 ? split_keys : kLatSplitKeys; }
+static inline int latent_max_splits(int max_kv_len, int split_keys) {
+  const int sk = latent_split_keys(split_keys);
+  return std::max(1, (max_kv_len + sk - 1) / sk);
+}
 
 }  // namespace pk
 
@@ -202,32 +356,56 @@ pegainfer_status_t pegainfer_latent_prep(const void* proj, int64_t proj_row_stri
   return (pegainfer_status_t)hipGetLastError();
 }
 
-int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, int32_t rank, int32_t max_kv_len) {
-  const int sp = latent_max_splits(max_kv_len);
+int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, int32_t rank, int32_t max_kv_len,
+                                             int32_t split_keys) {
+  const int sp = latent_max_splits(max_kv_len, split_keys);
   return sp <= 1 ? 0 : (int64_t)n_tokens * heads * sp * (rank + 2);
+}
+
+int32_t pegainfer_latent_attention_tiled_ok(int32_t rank, int32_t rot, int64_t page_stride, int64_t layer_off, int32_t dtype) {
+  const int Epad = (rank + rot + 31) & ~31;
+  const int nd = rank <= 64 ? 4 : rank <= 128 ? 8 : rank <= 256 ? 16 : 32;
+  return dtype == kDtBf16 && rank % 16 == 0 && rank <= 512 && rot % 8 == 0 && page_stride % 8 == 0 && layer_off % 8 == 0 &&
+         ((kTileRows + kTileKeys) * (Epad + 8) + nd * 16 * (kTileKeys + 8)) * 2 <= 160 * 1024;
 }
 
 pegainfer_status_t pegainfer_latent_attention(const float* qc, float* o_lat, const void* cache, int64_t page_stride,
                                               int64_t layer_off, int32_t page_size, const int32_t* positions,
                                               const int32_t* token_req, const int32_t* page_indptr,
                                               const int32_t* page_ids, int32_t heads, int32_t rank, int32_t rot,
-                                              float scale, int32_t n_tokens, int32_t max_kv_len, float* workspace,
-                                              int32_t dtype, pegainfer_stream_t stream) {
+                                              float scale, int32_t n_tokens, int32_t max_kv_len, int32_t split_keys,
+                                              float* workspace, const int32_t* tile_row0, const int32_t* tile_rows,
+                                              int32_t n_tiles, int32_t dtype, pegainfer_stream_t stream) {
   if (n_tokens <= 0 || heads <= 0) return 0;
-  const int sp = latent_max_splits(max_kv_len);
-  if (rank > kLatAcc * 256 || (sp > 1 && !workspace)) return (pegainfer_status_t)hipErrorInvalidValue;
-  const size_t smem = (size_t)(rank + rot + kLatKeys) * sizeof(float);
-  if (smem > 60000) return (pegainfer_status_t)hipErrorInvalidValue;
-  dim3 grid(n_tokens, heads, sp);
-  if (!by_dtype(dtype, [&](auto* t) {
-        using A = std::remove_pointer_t<decltype(t)>;
-        latent_attn_kernel<A><<<grid, 256, smem, as_stream(stream)>>>(qc, o_lat, static_cast<const A*>(cache), page_stride,
-                                                                       layer_off, page_size, positions, token_req, page_indptr,
-                                                                       page_ids, heads, rank, rot, scale, workspace, sp);
-      }))
-    return (pegainfer_status_t)hipErrorInvalidValue;
-  if (sp > 1)
-    latent_attn_merge_kernel<<<dim3(n_tokens, heads), 256, 0, as_stream(stream)>>>(o_lat, workspace, positions, heads, rank, sp);
+  const int sk = latent_split_keys(split_keys), sp = latent_max_splits(max_kv_len, split_keys);
+  if (sp > 1 && !workspace) return (pegainfer_status_t)hipErrorInvalidValue;
+  hipStream_t s = as_stream(stream);
+  if (tile_row0) {
+    if (!tile_rows || n_tiles <= 0 || !pegainfer_latent_attention_tiled_ok(rank, rot, page_stride, layer_off, dtype) ||
+        (reinterpret_cast<uintptr_t>(cache) & 15u))
+      return (pegainfer_status_t)hipErrorInvalidValue;
+    const uint16_t* c = static_cast<const uint16_t*>(cache);
+#define LAT_LAUNCH(ND) latent_attn_mfma_launch<ND>(qc, o_lat, c, page_stride, layer_off, page_size, positions, token_req, page_indptr, \
+                                                   page_ids, tile_row0, tile_rows, n_tiles, heads, rank, rot, scale, workspace, sp, sk, s)
+    if (rank <= 64) LAT_LAUNCH(4);
+    else if (rank <= 128) LAT_LAUNCH(8);
+    else if (rank <= 256) LAT_LAUNCH(16);
+    else LAT_LAUNCH(32);
+#undef LAT_LAUNCH
+  } else {
+    if (rank > kLatAcc * 256) return (pegainfer_status_t)hipErrorInvalidValue;
+    const size_t smem = (size_t)(rank + rot + kLatKeys) * sizeof(float);
+    if (smem > 60000) return (pegainfer_status_t)hipErrorInvalidValue;
+    dim3 grid(n_tokens, heads, sp);
+    if (!by_dtype(dtype, [&](auto* t) {
+          using A = std::remove_pointer_t<decltype(t)>;
+          latent_attn_kernel<A><<<grid, 256, smem, s>>>(qc, o_lat, static_cast<const A*>(cache), page_stride, layer_off, page_size,
+                                                        positions, token_req, page_indptr, page_ids, heads, rank, rot, scale,
+                                                        workspace, sp, sk);
+        }))
+      return (pegainfer_status_t)hipErrorInvalidValue;
+  }
+  if (sp > 1) latent_attn_merge_kernel<<<dim3(n_tokens, heads), 256, 0, s>>>(o_lat, workspace, positions, heads, rank, sp, sk);
   return (pegainfer_status_t)hipGetLastError();
 }
 

@@ -97,7 +97,7 @@ struct LayerW {
 struct Model {
   int device = 0, dtype = 0, D = 0, V = 0, max_requests = 0, num_pages = 0;
   float eps = 1e-5f;
-  bool plain_gemm = false, finalized = false;
+  bool plain_kernels = false, finalized = false;
   std::string err;
   std::vector<LayerCfg> layers;
   std::vector<LayerW> weights;          // indexed by owner layer
@@ -497,7 +497,7 @@ struct Model {
   }
   // Y[T, M] = X[T, K] W[M, K]^T in the model's storage type
   int linear(const void* W, const void* X, void* Y, int M, int T, int K, int epilogue = PEGAINFER_EPI_NONE) {
-    if (dtype == PEGAINFER_DTYPE_BF16 && !plain_gemm) {
+    if (dtype == PEGAINFER_DTYPE_BF16 && !plain_kernels) {
       gemm_cuda(static_cast<const Half*>(W), static_cast<const Half*>(X), static_cast<Half*>(Y), M, T, K, S());
       if (epilogue == PEGAINFER_EPI_RELU_SQ) DZ_K(pegainfer_relu_sq(Y, Y, (int64_t)M * T, dtype, S()));
       return 0;
@@ -544,7 +544,10 @@ struct Model {
     }
     const int W = (int)want.size();
     if (ensure_rows(T) || ensure_want((size_t)std::max(1, W))) return -1;
-    const int64_t ws_need = pegainfer_latent_attention_workspace((int)T, mx_heads, mx_rank, max_kv);
+    // decode-like steps (few rows) cut the keys finely so that one request's context spreads over many workgroups;
+    // prompt-sized steps have rows enough and only cut very long contexts
+    const int split_keys = T * (size_t)mx_heads <= 1024 ? 128 : 4096;
+    const int64_t ws_need = pegainfer_latent_attention_workspace((int)T, mx_heads, mx_rank, max_kv, split_keys);
     if ((size_t)ws_need > attn_ws_cap) {
       DZ_HIP(hipStreamSynchronize(stream));
       if (attn_ws) (void)hipFree(attn_ws);
@@ -560,8 +563,22 @@ struct Model {
       if (!st.ensure_capacity(&pool, st.seq_len + lens[i], kPageSize)) return set_error("step: page pool ran dry");   // cannot happen after the check above
       total_pages += st.pages.size();
     }
+    // row tiles of the matrix-core attention: per distinct head count, the flattened (token, head) rows cut into runs of
+    // <= 64 rows that stay inside one entry
+    std::vector<int> head_vals;
+    for (auto& c : layers)
+      if (std::find(head_vals.begin(), head_vals.end(), c.mx.heads) == head_vals.end()) head_vals.push_back(c.mx.heads);
+    std::vector<size_t> tile_off(head_vals.size()), tile_cnt(head_vals.size());
     const size_t o_tok = 0, o_pos = o_tok + T, o_req = o_pos + T, o_ind = o_req + T, o_want = o_ind + (size_t)n + 1,
-                 o_pages = o_want + (size_t)std::max(1, W), words = o_pages + total_pages;
+                 o_pages = o_want + (size_t)std::max(1, W);
+    size_t words = o_pages + total_pages;
+    for (size_t k = 0; k < head_vals.size(); ++k) {
+      size_t cnt = 0;
+      for (int i = 0; i < n; ++i) cnt += ((size_t)lens[i] * head_vals[k] + 63) / 64;
+      tile_off[k] = words;
+      tile_cnt[k] = cnt;
+      words += 2 * cnt;
+    }
     if (words > cap_meta) {
       DZ_HIP(hipStreamSynchronize(stream));
       if (meta_host) (void)hipHostFree(meta_host);
@@ -589,6 +606,18 @@ struct Model {
       }
       mh[o_ind + n] = (int32_t)pg;
       for (int i = 0; i < W; ++i) mh[o_want + i] = want[i];
+      for (size_t k = 0; k < head_vals.size(); ++k) {
+        const int Hk = head_vals[k];
+        size_t at = 0, tok0 = 0;
+        for (int i = 0; i < n; ++i) {
+          const int rows = lens[i] * Hk;
+          for (int r0 = 0; r0 < rows; r0 += 64, ++at) {
+            mh[tile_off[k] + at] = (int32_t)(tok0 * Hk) + r0;
+            mh[tile_off[k] + tile_cnt[k] + at] = std::min(64, rows - r0);
+          }
+          tok0 += (size_t)lens[i];
+        }
+      }
     }
     DZ_HIP(hipEventRecord(ev0, stream));
     DZ_HIP(hipMemcpyAsync(meta_dev, meta_host, words * 4, hipMemcpyHostToDevice, stream));
@@ -635,8 +664,14 @@ struct Model {
       } else {
         DZ_HIP(hipMemsetAsync(qc, 0, T * (size_t)m.heads * E * 4, stream));
       }
-      DZ_K(pegainfer_latent_attention(qc, olat, cache, page_stride, c.cache_off, kPageSize, d_pos, d_req, d_ind, d_pages,
-                                      m.heads, m.rank, m.rot, m.scale, Ti, max_kv, attn_ws, dtype, S()));
+      {
+        const size_t hk = std::find(head_vals.begin(), head_vals.end(), m.heads) - head_vals.begin();
+        const bool tiled = !plain_kernels && pegainfer_latent_attention_tiled_ok(m.rank, m.rot, page_stride, c.cache_off, dtype);
+        DZ_K(pegainfer_latent_attention(qc, olat, cache, page_stride, c.cache_off, kPageSize, d_pos, d_req, d_ind, d_pages,
+                                        m.heads, m.rank, m.rot, m.scale, Ti, max_kv, split_keys, attn_ws,
+                                        tiled ? md + tile_off[hk] : nullptr, tiled ? md + tile_off[hk] + tile_cnt[hk] : nullptr,
+                                        (int)tile_cnt[hk], dtype, S()));
+      }
       {  // value up-projection per head + sigmoid gate
         pegainfer_gemm_desc d{};
         d.x = olat; d.w = w.uv; d.y = attn;
@@ -849,6 +884,6 @@ int32_t pegainfer_duguzen_debug_hidden(pegainfer_duguzen_t m, int32_t layer_run,
 }
 float pegainfer_duguzen_last_step_ms(pegainfer_duguzen_t m) { return M(m)->last_step_ms; }
 int64_t pegainfer_duguzen_weight_bytes(pegainfer_duguzen_t m) { return M(m)->weight_bytes; }
-int32_t pegainfer_duguzen_set_plain_gemm(pegainfer_duguzen_t m, int32_t on) { M(m)->plain_gemm = on != 0; return 0; }
+int32_t pegainfer_duguzen_set_plain_kernels(pegainfer_duguzen_t m, int32_t on) { M(m)->plain_kernels = on != 0; return 0; }
 
 }  // extern "C"

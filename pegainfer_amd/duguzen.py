@@ -69,8 +69,8 @@ class DuguzenEngine:
         self._chk(self.lib.pegainfer_duguzen_finalize(self.h), "finalize")
         return self
 
-    def set_plain_gemm(self, on=True):
-        self.lib.pegainfer_duguzen_set_plain_gemm(self.h, int(bool(on)))
+    def set_plain_kernels(self, on=True):
+        self.lib.pegainfer_duguzen_set_plain_kernels(self.h, int(bool(on)))
 
     # ---- requests ----
     def new_request(self):

@@ -98,17 +98,30 @@ def latent_prep(proj, dkv_offset, c_norm_w, eps, inv_freq, rot_dims, positions, 
                                          _stream()), "latent_prep")
 
 
+def row_tiles(lens, heads, device="cuda"):
+    """the flattened (token, head) rows of a step with entries of `lens` tokens, cut into runs of <= 64 rows inside one entry"""
+    row0, rows, at = [], [], 0
+    for n in lens:
+        for r in range(0, n * heads, 64):
+            row0.append(at * heads + r)
+            rows.append(min(64, n * heads - r))
+        at += n
+    return (torch.tensor(row0, dtype=torch.int32, device=device), torch.tensor(rows, dtype=torch.int32, device=device))
+
+
 def latent_attention(qc, cache, page_stride, layer_off, page_size, positions, token_req, page_indptr, page_ids, rank, rot,
-                     scale, max_kv_len):
-    """qc fp32 [T, heads, rank + rot] -> o_lat fp32 [T, heads, rank]"""
+                     scale, max_kv_len, split_keys=0, tiles=None):
+    """qc fp32 [T, heads, rank + rot] -> o_lat fp32 [T, heads, rank]; tiles = row_tiles(...) selects the matrix-core form"""
     T, H, E = qc.shape
     assert E == rank + rot and qc.dtype == torch.float32
     o = torch.empty((T, H, rank), dtype=torch.float32, device=qc.device)
-    n = ffi.lib().pegainfer_latent_attention_workspace(T, H, rank, max_kv_len)
+    n = ffi.lib().pegainfer_latent_attention_workspace(T, H, rank, max_kv_len, split_keys)
     ws = torch.empty(max(int(n), 1), dtype=torch.float32, device=qc.device)
+    t0, tr = tiles if tiles is not None else (None, None)
     _chk(ffi.lib().pegainfer_latent_attention(_p(qc), _p(o), _p(cache), page_stride, layer_off, page_size, _p(positions),
                                               _p(token_req), _p(page_indptr), _p(page_ids), H, rank, rot, float(scale), T,
-                                              max_kv_len, _p(ws), _dt(cache), _stream()), "latent_attention")
+                                              max_kv_len, split_keys, _p(ws), _p(t0), _p(tr), 0 if t0 is None else t0.numel(),
+                                              _dt(cache), _stream()), "latent_attention")
     return o
 
 

@@ -46,7 +46,7 @@ def test_whole_prompt_every_position_and_every_layer(name, dtype):
         assert np.abs(H[i] - t.numpy()).max() < (2e-5 if dtype == "float32" else 4e-2) * scale, i
     if dtype == "bfloat16":          # the tuned GEMM routes and the plain tile kernel agree to rounding
         eng.drop_request(r)
-        eng.set_plain_gemm(True)
+        eng.set_plain_kernels(True)
         r = eng.new_request()
         check(eng.step([(r, toks)], want=list(range(len(toks)))), ref, dtype)
     eng.close()

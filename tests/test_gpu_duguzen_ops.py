@@ -243,3 +243,72 @@ def test_latent_attention_rows_of_several_requests():
     for i, (q, p) in enumerate(rows):
         s = torch.einsum("he,je->hj", qc[i].double(), ent[q][:p + 1].double()) * 0.5
         assert (o[i].double() - torch.softmax(s, -1) @ ent[q][:p + 1, :r].double()).abs().max() < 2e-5
+
+
+@pytest.mark.parametrize("split_keys", [0, 128])
+@pytest.mark.parametrize("shape", [(3, 32, 8, [70, 1, 9]), (8, 64, 32, [300, 2]), (5, 16, 16, [13, 13, 1, 1]), (16, 128, 64, [5, 40])])
+def test_latent_attention_matrix_core_form(shape, split_keys):
+    """the tiled bf16 form against the direct softmax: several requests in one launch, portions that start deep inside a
+    context, tiles that end inside an entry, key splits; q and the weights are rounded to bf16 inside, hence the tolerance"""
+    from pegainfer_amd import ops_blocks as B
+    H, r, dr, lens = shape
+    g = torch.Generator().manual_seed(H * 100 + r)
+    E, ps = r + dr, 16
+    starts = [0 if i % 2 == 0 else 137 for i in range(len(lens))]          # odd entries continue a context of 137 tokens
+    ctx = [s + n for s, n in zip(starts, lens)]
+    ent = [C.bf16_round(torch.randn(n, E, generator=g) * 0.7) for n in ctx]
+    npages = [(n + ps - 1) // ps for n in ctx]
+    pool = torch.zeros(sum(npages) + 2, ps, E)
+    order = np.random.default_rng(H).permutation(sum(npages) + 2)
+    page_lists, at = [], 0
+    for e, k in zip(ent, npages):
+        pl = [int(x) for x in order[at:at + k]]
+        at += k
+        for j in range(len(e)):
+            pool[pl[j // ps], j % ps] = e[j]
+        page_lists.append(pl)
+    indptr = np.cumsum([0] + npages).astype(np.int32)
+    pos = [s + k for s, n in zip(starts, lens) for k in range(n)]
+    req = [i for i, n in enumerate(lens) for _ in range(n)]
+    T = len(pos)
+    qc = torch.randn(T, H, E, generator=g)
+    assert ffi_ok(B, r, dr, ps * E)
+    args = (dev(pool, torch.bfloat16), ps * E, 0, ps, torch.tensor(pos, dtype=torch.int32).cuda(), torch.tensor(req, dtype=torch.int32).cuda(),
+            torch.tensor(indptr).cuda(), torch.tensor(sum(page_lists, []), dtype=torch.int32).cuda(), r, dr, 0.25, max(ctx))
+    o = B.latent_attention(dev(qc), *args, split_keys=split_keys, tiles=B.row_tiles(lens, H)).cpu()
+    plain = B.latent_attention(dev(qc), *args, split_keys=split_keys).cpu()
+    for i in range(T):
+        e = ent[req[i]][:pos[i] + 1].double()
+        ref = torch.softmax(torch.einsum("he,je->hj", qc[i].double(), e) * 0.25, -1) @ e[:, :r]
+        assert (plain[i].double() - ref).abs().max() < 2e-5, i
+        assert (o[i].double() - ref).abs().max() < 2.5e-2, (i, pos[i], float((o[i].double() - ref).abs().max()))
+    assert float((o - plain).abs().mean()) < 2e-3
+
+
+def ffi_ok(B, r, dr, page_stride):
+    from pegainfer_amd import ffi
+    return ffi.lib().pegainfer_latent_attention_tiled_ok(r, dr, page_stride, 0, 0) == 1
+
+
+def test_matrix_core_form_sees_a_far_key_and_masks_an_unseen_one():
+    from pegainfer_amd import ops_blocks as B
+    for far in (0, 31, 32, 127, 128, 700):
+        g = torch.Generator().manual_seed(far)
+        n, H, r, dr, ps = 800, 8, 16, 16, 16
+        E = r + dr
+        entries = C.bf16_round(torch.randn(n, E, generator=g) * 0.2)
+        probe = torch.zeros(E)
+        probe[3], probe[r + 1] = 8.0, 8.0
+        entries[far] = probe
+        cache, pages = _paged(entries, ps, torch.bfloat16, perm_seed=far)
+        lo = max(far - 1, 0)
+        T = n - lo                                       # one portion: positions lo .. n-1
+        qc = torch.zeros(T, H, E)
+        qc[:, :, 3] = qc[:, :, r + 1] = 4.0
+        o = B.latent_attention(dev(qc), cache, ps * E, 0, ps, torch.arange(lo, n, dtype=torch.int32).cuda(),
+                               torch.zeros(T, dtype=torch.int32).cuda(), torch.tensor([0, len(pages)], dtype=torch.int32).cuda(),
+                               pages, r, dr, 1.0, n, split_keys=128, tiles=B.row_tiles([T], H)).cpu()
+        seen = o[far - lo:]
+        assert (seen - probe[:r]).abs().max() < 2e-2, far
+        if far > 0:
+            assert float(o[0][:, 3].abs().max()) < 1.0
