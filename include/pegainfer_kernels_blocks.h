@@ -47,8 +47,11 @@ pegainfer_status_t pegainfer_silu_mul_rows(const void* gate_up, void* out, int32
  * Dense form (tile_group == NULL): `rows` rows in each of `groups` groups.
  * Grouped form: a device-side table of row tiles, each of <= 64 consecutive POSITIONS of a sorted list that belong to
  * one group (expert); positions map to x / y rows through x_row_index / y_row_index (NULL = identity).  Tiles beyond
- * *n_tiles exit; the grid is max_tiles wide.  The k order of every output is fixed, so a row's result does not depend
- * on what else is in the launch. */
+ * *n_tiles exit; the grid is max_tiles wide.
+ * Three kernels behind one entry: an fp32-FMA tile kernel (any sizes and strides, both storage types), a matrix-core tile
+ * kernel (bf16 weights with contiguous k in 16-byte chunks; an fp32 x is rounded to bf16 as it is staged) and a few-rows
+ * form that streams the weights once (<= 8 rows per tile: decode).  In each the k order of an output is fixed, so a row's
+ * result does not depend on what else is in the launch; which kernel runs depends on the launch's shape. */
 enum { PEGAINFER_EPI_NONE = 0, PEGAINFER_EPI_RELU_SQ = 1, PEGAINFER_EPI_SIGMOID_GATE = 2 };
 typedef struct {
   const void* x;
@@ -70,6 +73,8 @@ typedef struct {
   const void* gate;
   int32_t gate_dtype;
   int64_t gate_row_stride;
+  int32_t max_tile_rows;     /* grouped form: an upper bound of tile_rows the caller knows (0 = 64) */
+  int32_t plain;             /* != 0: always the fp32-FMA tile kernel (exact products of the stored values) */
 } pegainfer_gemm_desc;
 pegainfer_status_t pegainfer_gemm_strided(const pegainfer_gemm_desc* d, pegainfer_stream_t stream);
 

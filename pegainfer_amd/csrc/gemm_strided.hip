@@ -9,6 +9,8 @@
 // tile it lands in, the batch or the group sizes).  Operand storage (bf16 or fp32) is a template parameter, so the bf16
 // instance multiplies exact fp32 images of bf16 values and the fp32 instance is plain fp32 FMA - no reduced-precision
 // matrix mode.
+#include <type_traits>
+
 #include "common.h"
 #include "typed.h"
 #include "pegainfer_kernels_blocks.h"
@@ -93,10 +95,211 @@ __global__ __launch_bounds__(256) void gemm_strided_kernel(pegainfer_gemm_desc d
   }
 }
 
+
+// ------------------------------------------------------------------ matrix-core form (bf16 weights, k contiguous)
+// Same 64 x 64 tile and the same addressing (groups, gathered rows, tile table), K in slices of 64 staged as bf16, four waves
+// in a 2 x 2 arrangement, each 2 x 2 blocks of v_mfma_f32_16x16x32_bf16.  fp32 x (the attention output in front of the value
+// up-projection) is rounded to bf16 while it is staged.  Needs 16-byte chunks: K % 8 == 0, strides % 8 == 0, aligned bases.
+constexpr int MK = 64, MS = MK + 8;
+
+__device__ __forceinline__ u32x4 stage8(const uint16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ u32x4 stage8(const float* p) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+  return u32x4{pack_bf2(a.x, a.y), pack_bf2(a.z, a.w), pack_bf2(b.x, b.y), pack_bf2(b.z, b.w)};
+}
+
+template <typename TX, typename TY, typename TG>
+__global__ __launch_bounds__(256) void gemm_strided_mfma_kernel(pegainfer_gemm_desc d) {
+  __shared__ __align__(16) uint16_t xs[GT * MS];
+  __shared__ __align__(16) uint16_t ws[GM * MS];
+  __shared__ int xrow[GT], yrow[GT];
+  int g, row0, nrows;
+  if (d.tile_group) {
+    if ((int)blockIdx.x >= *d.n_tiles) return;
+    g = d.tile_group[blockIdx.x];
+    row0 = d.tile_row0[blockIdx.x];
+    nrows = d.tile_rows[blockIdx.x];
+  } else {
+    g = blockIdx.z;
+    row0 = blockIdx.x * GT;
+    nrows = min(GT, d.rows - row0);
+  }
+  const int m0 = blockIdx.y * GM;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l15 = lane & 15, gq = lane >> 4;
+  if (tid < GT) {
+    const int p = row0 + tid;
+    xrow[tid] = tid < nrows ? (d.x_row_index ? d.x_row_index[p] : p) : -1;
+    yrow[tid] = tid < nrows ? (d.y_row_index ? d.y_row_index[p] : p) : -1;
+  }
+  __syncthreads();
+  const TX* X = static_cast<const TX*>(d.x) + (int64_t)g * d.x_group_stride;
+  const uint16_t* W = static_cast<const uint16_t*>(d.w) + (int64_t)g * d.w_group_stride;
+  const int wr = (wave & 1) * 32, wm = (wave >> 1) * 32;
+  f32x4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int k0 = 0; k0 < d.k; k0 += MK) {
+#pragma unroll
+    for (int c = tid; c < GT * (MK / 8); c += 256) {
+      const int r = c >> 3, kk = k0 + (c & 7) * 8;
+      const int src = xrow[r];
+      *reinterpret_cast<u32x4*>(xs + r * MS + (c & 7) * 8) = (src >= 0 && kk < d.k) ? stage8(X + (int64_t)src * d.x_row_stride + kk) : zero;
+      *reinterpret_cast<u32x4*>(ws + r * MS + (c & 7) * 8) =
+          (m0 + r < d.m && kk < d.k) ? stage8(W + (int64_t)(m0 + r) * d.w_m_stride + kk) : zero;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < MK; ks += 32) {
+      bf16x8_t a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(ws + (wm + i * 16 + l15) * MS + ks + gq * 8));
+        b[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xs + (wr + i * 16 + l15) * MS + ks + gq * 8));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int r = wr + j * 16 + l15;
+    const int dst = yrow[r];
+    if (dst < 0) continue;
+    float scale = 1.f;
+    if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
+      scale = sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + wm + i * 16 + gq * 4 + e;
+        if (m >= d.m) continue;
+        float v = acc[i][j][e];
+        if (d.epilogue == PEGAINFER_EPI_RELU_SQ) { v = fmaxf(v, 0.f); v *= v; }
+        else if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE) v *= scale;
+        st(Y + (int64_t)dst * d.y_row_stride + m, v);
+      }
+  }
+}
+
+// ------------------------------------------------------------------ few-rows form (decode)
+// At most R rows per tile (a decode step's tokens, or the pairs one expert received): the weights are streamed once with
+// 16-byte loads, the rows wait in LDS as fp32, a wave owns one output at a time (lanes over k, butterfly sum), 32 outputs per
+// workgroup.  fp32 arithmetic for both storage types; the k order of an output is fixed by K alone.
+constexpr int kRowsFormOutputs = 32;
+
+template <typename TX, typename TW, typename TY, typename TG, int R>
+__global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_desc d) {
+  extern __shared__ float xr[];    // [R][K]
+  __shared__ int xrow[R], yrow[R];
+  int g, row0, nrows;
+  if (d.tile_group) {
+    if ((int)blockIdx.x >= *d.n_tiles) return;
+    g = d.tile_group[blockIdx.x];
+    row0 = d.tile_row0[blockIdx.x];
+    nrows = min(R, d.tile_rows[blockIdx.x]);
+  } else {
+    g = blockIdx.z;
+    row0 = blockIdx.x * R;
+    nrows = min(R, d.rows - row0);
+  }
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  if (tid < R) {
+    const int p = row0 + tid;
+    xrow[tid] = tid < nrows ? (d.x_row_index ? d.x_row_index[p] : p) : -1;
+    yrow[tid] = tid < nrows ? (d.y_row_index ? d.y_row_index[p] : p) : -1;
+  }
+  __syncthreads();
+  const TX* X = static_cast<const TX*>(d.x) + (int64_t)g * d.x_group_stride;
+  const TW* W = static_cast<const TW*>(d.w) + (int64_t)g * d.w_group_stride;
+  const int K = d.k;
+  for (int i = tid; i < R * K; i += 256) {
+    const int r = i / K, k = i - r * K;
+    xr[i] = xrow[r] >= 0 ? ld(X + (int64_t)xrow[r] * d.x_row_stride + k) : 0.f;
+  }
+  __syncthreads();
+  TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
+  const int m_base = blockIdx.y * kRowsFormOutputs;
+  for (int mi = wave; mi < kRowsFormOutputs; mi += 4) {
+    const int m = m_base + mi;
+    if (m >= d.m) break;
+    const TW* wrow = W + (int64_t)m * d.w_m_stride;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+#pragma unroll 2
+    for (int k = lane * 8; k < K; k += 512) {
+      float wv[8];
+      Vec8<TW>::load(wrow + k, wv);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const f32x4 xa = *reinterpret_cast<const f32x4*>(xr + r * K + k), xb = *reinterpret_cast<const f32x4*>(xr + r * K + k + 4);
+        float a = acc[r];
+        a = fmaf(wv[0], xa.x, a); a = fmaf(wv[1], xa.y, a); a = fmaf(wv[2], xa.z, a); a = fmaf(wv[3], xa.w, a);
+        a = fmaf(wv[4], xb.x, a); a = fmaf(wv[5], xb.y, a); a = fmaf(wv[6], xb.z, a); a = fmaf(wv[7], xb.w, a);
+        acc[r] = a;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (yrow[r] < 0) continue;
+        float v = acc[r];
+        if (d.epilogue == PEGAINFER_EPI_RELU_SQ) { v = fmaxf(v, 0.f); v *= v; }
+        else if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
+          v *= sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
+        st(Y + (int64_t)yrow[r] * d.y_row_stride + m, v);
+      }
+    }
+  }
+}
+
+template <typename TX, typename TW, typename TY, typename TG, int R>
+static void rows_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
+  auto kern = &gemm_strided_rows_kernel<TX, TW, TY, TG, R>;
+  // 150 KB of rows at most (checked by the caller) next to the kernel's few static words
+  static const bool once = (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                152 * 1024), true);
+  (void)once;
+  dim3 grid(d.tile_group ? d.max_tiles : ceil_div(d.rows, R), ceil_div(d.m, kRowsFormOutputs), d.tile_group ? 1 : d.groups);
+  kern<<<grid, 256, (size_t)R * d.k * sizeof(float), s>>>(d);
+}
+
+static inline bool chunks_ok(const pegainfer_gemm_desc& d) {
+  auto a16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  return d.w_k_stride == 1 && (d.k & 7) == 0 && (d.x_row_stride & 7) == 0 && (d.x_group_stride & 7) == 0 &&
+         (d.w_m_stride & 7) == 0 && (d.w_group_stride & 7) == 0 && a16(d.x) && a16(d.w);
+}
+
 template <typename TX, typename TW, typename TY>
 static void gemm_strided_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
   dim3 grid(d.tile_group ? d.max_tiles : ceil_div(d.rows, GT), ceil_div(d.m, GM), d.tile_group ? 1 : d.groups);
-  if (d.gate_dtype == kDtF32) gemm_strided_kernel<TX, TW, TY, float><<<grid, 256, 0, s>>>(d);
+  const bool gate32 = d.gate_dtype == kDtF32;
+  if (!d.plain && chunks_ok(d)) {
+    // few rows per tile: stream the weights once (both storage types, fp32 arithmetic)
+    const int tr = d.tile_group ? (d.max_tile_rows > 0 ? d.max_tile_rows : GT) : d.rows;
+    const int R = tr <= 1 ? 1 : tr <= 4 ? 4 : tr <= 8 ? 8 : 0;
+    if (R && (size_t)R * d.k * sizeof(float) <= 150 * 1024) {
+      if (gate32) { if (R == 1) rows_form_launch<TX, TW, TY, float, 1>(d, s); else if (R == 4) rows_form_launch<TX, TW, TY, float, 4>(d, s); else rows_form_launch<TX, TW, TY, float, 8>(d, s); }
+      else { if (R == 1) rows_form_launch<TX, TW, TY, uint16_t, 1>(d, s); else if (R == 4) rows_form_launch<TX, TW, TY, uint16_t, 4>(d, s); else rows_form_launch<TX, TW, TY, uint16_t, 8>(d, s); }
+      return;
+    }
+    if constexpr (std::is_same<TW, uint16_t>::value) {   // bf16 weights: the matrix cores
+      if (gate32) gemm_strided_mfma_kernel<TX, TY, float><<<grid, 256, 0, s>>>(d);
+      else gemm_strided_mfma_kernel<TX, TY, uint16_t><<<grid, 256, 0, s>>>(d);
+      return;
+    }
+  }
+  if (gate32) gemm_strided_kernel<TX, TW, TY, float><<<grid, 256, 0, s>>>(d);
   else gemm_strided_kernel<TX, TW, TY, uint16_t><<<grid, 256, 0, s>>>(d);
 }
 

@@ -24,7 +24,6 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
-#include <random>
 #include <string>
 #include <vector>
 
@@ -82,7 +81,9 @@ struct LayerCfg {
   int owner = 0;
   int64_t cache_off = 0;   // element offset of this layer run's slice inside a page
   int entry() const { return mx.rank + mx.rot; }
-  int proj_rows() const { return mx.heads * (mx.nope + mx.rot) + mx.rank + mx.rot + mx.heads; }
+  // rows of the stacked projection [q ; dkv ; g], padded with zero rows to a multiple of 8 so that every row of its output
+  // starts on a 16-byte boundary
+  int proj_rows() const { return (mx.heads * (mx.nope + mx.rot) + mx.rank + mx.rot + mx.heads + 7) & ~7; }
 };
 struct Norm { void *w = nullptr, *b = nullptr, *alpha = nullptr; };
 struct LayerW {
@@ -321,8 +322,18 @@ struct Model {
     return 0;
   }
   int fill_synthetic(uint64_t seed, float std) {
-    std::mt19937_64 rng(seed);
-    std::normal_distribution<float> g(0.f, 1.f);
+    // splitmix64 stream; a unit-variance value = sum of four uniforms, centred and scaled (cheap, and enough for weights)
+    uint64_t state = seed * 0x9E3779B97F4A7C15ull + 0x1234567ull;
+    auto g = [&state](int) {
+      state += 0x9E3779B97F4A7C15ull;
+      uint64_t z = state;
+      z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+      z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+      z ^= z >> 31;
+      const float u = (float)(z & 0xFFFF) + (float)((z >> 16) & 0xFFFF) + (float)((z >> 32) & 0xFFFF) + (float)(z >> 48);
+      return (u * (1.0f / 65536.0f) - 2.0f) * 1.7320508f;
+    };
+    int rng = 0;
     for (auto& t : tensor_list()) {
       const std::string& n = t.first;
       std::vector<uint16_t>& v = staged[n];
@@ -382,9 +393,20 @@ struct Model {
         std::vector<uint16_t> st(*q);
         st.insert(st.end(), dkv->begin(), dkv->end());
         st.insert(st.end(), g->begin(), g->end());
+        st.resize((size_t)c.proj_rows() * D, 0);
         if (upload(&w.proj, st.data(), st.size())) return -1;
       }
-      if (up(&w.cnorm, p + ".mix.dkv.norm", m.rank) || up(&w.uk, p + ".mix.uk", (int64_t)m.heads * m.nope * m.rank) ||
+      {  // key up-projection stored transposed per head, [heads][rank][nope]: the absorb GEMM reads it with k contiguous
+        const auto* uk = need(p + ".mix.uk", (int64_t)m.heads * m.nope * m.rank);
+        if (!uk) return -1;
+        std::vector<uint16_t> tr(uk->size());
+        for (int hh = 0; hh < m.heads; ++hh)
+          for (int dd = 0; dd < m.nope; ++dd)
+            for (int rr = 0; rr < m.rank; ++rr)
+              tr[((size_t)hh * m.rank + rr) * m.nope + dd] = (*uk)[((size_t)hh * m.nope + dd) * m.rank + rr];
+        if (upload(&w.uk, tr.data(), tr.size())) return -1;
+      }
+      if (up(&w.cnorm, p + ".mix.dkv.norm", m.rank) ||
           up(&w.uv, p + ".mix.uv", (int64_t)m.heads * m.vdim * m.rank) || up(&w.o, p + ".mix.o", (int64_t)D * m.heads * m.vdim))
         return -1;
       {  // rotation frequencies base^(-2i/dims), rounded once to fp32
@@ -508,6 +530,7 @@ struct Model {
     d.m = M; d.k = K; d.rows = T; d.groups = 1;
     d.x_row_stride = K; d.w_m_stride = K; d.w_k_stride = 1; d.y_row_stride = M;
     d.epilogue = epilogue;
+    d.plain = plain_kernels;
     DZ_K(pegainfer_gemm_strided(&d, S()));
     return 0;
   }
@@ -658,8 +681,9 @@ struct Model {
         d.x_dtype = d.w_dtype = dtype; d.y_dtype = PEGAINFER_DTYPE_F32;
         d.m = m.rank; d.k = m.nope; d.rows = Ti; d.groups = m.heads;
         d.x_row_stride = Mp; d.x_group_stride = m.nope + m.rot;
-        d.w_m_stride = 1; d.w_k_stride = m.rank; d.w_group_stride = (int64_t)m.nope * m.rank;
+        d.w_m_stride = m.nope; d.w_k_stride = 1; d.w_group_stride = (int64_t)m.nope * m.rank;
         d.y_row_stride = (int64_t)m.heads * E; d.y_group_stride = E;
+        d.plain = plain_kernels;
         DZ_K(pegainfer_gemm_strided(&d, S()));
       } else {
         DZ_HIP(hipMemsetAsync(qc, 0, T * (size_t)m.heads * E * 4, stream));
@@ -684,6 +708,7 @@ struct Model {
         d.gate = static_cast<const uint8_t*>(proj) + (size_t)(qrow + E) * esize();
         d.gate_dtype = dtype;
         d.gate_row_stride = Mp;
+        d.plain = plain_kernels;
         DZ_K(pegainfer_gemm_strided(&d, S()));
       }
       if (linear(w.o, attn, y, D, Ti, m.heads * m.vdim)) return -1;
@@ -740,6 +765,8 @@ struct Model {
     d.y_row_stride = 2 * f.ff;
     d.tile_group = t_group; d.tile_row0 = t_row0; d.tile_rows = t_rows; d.n_tiles = n_tiles; d.max_tiles = (P + 63) / 64 + f.experts;
     d.x_row_index = pos_row;
+    d.max_tile_rows = std::min(T, 64);   // a row chooses distinct experts: an expert never gets more pairs than there are rows
+    d.plain = plain_kernels;
     DZ_K(pegainfer_gemm_strided(&d, S()));
     DZ_K(pegainfer_silu_mul_rows(gu, act, f.ff, P, dtype, S()));
     pegainfer_gemm_desc e{};
@@ -750,6 +777,8 @@ struct Model {
     e.y_row_stride = D;
     e.tile_group = t_group; e.tile_row0 = t_row0; e.tile_rows = t_rows; e.n_tiles = n_tiles; e.max_tiles = d.max_tiles;
     e.y_row_index = pos_pair;
+    e.max_tile_rows = d.max_tile_rows;
+    e.plain = plain_kernels;
     DZ_K(pegainfer_gemm_strided(&e, S()));
     DZ_K(pegainfer_route_combine(ypairs, route_w, y, D, f.top, T, dtype, S()));
     return 0;

@@ -25,10 +25,22 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
   float* gs = sm + 2 * E;   // [G] group scores
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const A* x = h + (size_t)row * d;
+  const bool vec = (d & 7) == 0 && aligned16(x) && aligned16(wr);
   for (int e = wave; e < E; e += 4) {
     const A* w = wr + (size_t)e * d;
     float a = 0.f;
-    for (int i = lane; i < d; i += 64) a = fmaf(ld(x + i), ld(w + i), a);
+    if (vec) {
+#pragma unroll 2
+      for (int i = lane * 8; i < d; i += 512) {
+        float xv[8], wv[8];
+        Vec8<A>::load(x + i, xv);
+        Vec8<A>::load(w + i, wv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a = fmaf(xv[k], wv[k], a);
+      }
+    } else {
+      for (int i = lane; i < d; i += 64) a = fmaf(ld(x + i), ld(w + i), a);
+    }
     a = wave_sum(a);
     if (lane == 0) {
       const float sc = sigmoid_f(a);

@@ -21,6 +21,26 @@ inline bool by_dtype(int dtype, F&& fn) {
   return false;
 }
 
+// eight consecutive stored values widened to fp32 (16-byte aligned for bf16, 32-byte span for fp32)
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<uint16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const uint16_t* p, float* o) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(p);
+    o[0] = bf_lo(v.x); o[1] = bf_hi(v.x); o[2] = bf_lo(v.y); o[3] = bf_hi(v.y);
+    o[4] = bf_lo(v.z); o[5] = bf_hi(v.z); o[6] = bf_lo(v.w); o[7] = bf_hi(v.w);
+  }
+};
+template <>
+struct Vec8<float> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const float* p, float* o) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+};
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 }  // namespace pk

@@ -33,7 +33,7 @@ class GemmDesc(ctypes.Structure):
                 ("n_tiles", ctypes.c_void_p), ("max_tiles", ctypes.c_int32),
                 ("x_row_index", ctypes.c_void_p), ("y_row_index", ctypes.c_void_p),
                 ("epilogue", ctypes.c_int32), ("gate", ctypes.c_void_p), ("gate_dtype", ctypes.c_int32),
-                ("gate_row_stride", ctypes.c_int64)]
+                ("gate_row_stride", ctypes.c_int64), ("max_tile_rows", ctypes.c_int32), ("plain", ctypes.c_int32)]
 
 
 def embed_f32(embed, token_ids_u32):
@@ -79,13 +79,14 @@ def gemm_strided(desc):
     _chk(ffi.lib().pegainfer_gemm_strided(ctypes.addressof(desc), _stream()), "gemm_strided")
 
 
-def linear(x, w, out_dtype=None, epilogue=EPI_NONE):
-    """y[T, M] = x[T, K] w[M, K]^T on the strided tile kernel (any sizes, bf16 or fp32 operands, fp32 accumulation)"""
+def linear(x, w, out_dtype=None, epilogue=EPI_NONE, plain=False):
+    """y[T, M] = x[T, K] w[M, K]^T through pegainfer_gemm_strided (any sizes, bf16 or fp32 operands, fp32 accumulation);
+    plain = the fp32-FMA tile kernel whatever the shape"""
     T, K = x.shape
     M = w.shape[0]
     y = torch.empty((T, M), dtype=out_dtype or x.dtype, device=x.device)
     d = GemmDesc(x=_p(x), w=_p(w), y=_p(y), x_dtype=_dt(x), w_dtype=_dt(w), y_dtype=_dt(y), m=M, k=K, rows=T, groups=1,
-                 x_row_stride=K, w_m_stride=K, w_k_stride=1, y_row_stride=M, epilogue=epilogue)
+                 x_row_stride=K, w_m_stride=K, w_k_stride=1, y_row_stride=M, epilogue=epilogue, plain=int(plain))
     gemm_strided(d)
     return y
 

@@ -312,3 +312,38 @@ def test_matrix_core_form_sees_a_far_key_and_masks_an_unseen_one():
         assert (seen - probe[:r]).abs().max() < 2e-2, far
         if far > 0:
             assert float(o[0][:, 3].abs().max()) < 1.0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_strided_gemm_forms_agree(dtype):
+    """the few-rows form (<= 8 rows), the matrix-core tile form (bf16 weights) and the fp32-FMA tile form compute the same
+    products of the stored values; only the order of the fp32 sums differs"""
+    from pegainfer_amd import ops_blocks as B
+    td = DT[dtype]
+    g = torch.Generator().manual_seed(7)
+    for (T, M, K) in [(1, 96, 128), (4, 33, 256), (7, 40, 64), (8, 200, 1024), (9, 40, 64), (70, 130, 192), (64, 64, 64), (200, 72, 320)]:
+        x, w = C.bf16_round(torch.randn(T, K, generator=g)), C.bf16_round(torch.randn(M, K, generator=g))
+        ref = x.double() @ w.double().T
+        for epi in (B.EPI_NONE, B.EPI_RELU_SQ):
+            want = ref if epi == B.EPI_NONE else torch.relu(ref) ** 2
+            fast = B.linear(dev(x, td), dev(w, td), out_dtype=torch.float32, epilogue=epi).cpu()
+            plain = B.linear(dev(x, td), dev(w, td), out_dtype=torch.float32, epilogue=epi, plain=True).cpu()
+            tol = 2e-5 * K * (1 if epi == B.EPI_NONE else 10)
+            assert (fast.double() - want).abs().max() < tol and (plain.double() - want).abs().max() < tol, (T, M, K, epi)
+    # grouped rows with a small bound on the rows per tile: the few-rows form walks the same tile table
+    rows, top, E, d, ff = 5, 2, 6, 64, 24
+    expert = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(rows)]).int()
+    pos_pair, pos_row, tg, t0, tr, nt, max_tiles = B.route_sort(expert.cuda(), E)
+    x, w = C.bf16_round(torch.randn(rows, d, generator=g)), C.bf16_round(torch.randn(E, ff, d, generator=g))
+    xd, wd = dev(x, td), dev(w, td)
+    outs = []
+    for plain in (0, 1):
+        y = torch.zeros(rows * top, ff, device="cuda")
+        B.gemm_strided(B.GemmDesc(x=xd.data_ptr(), w=wd.data_ptr(), y=y.data_ptr(), x_dtype=B._dt(xd), w_dtype=B._dt(wd), y_dtype=1,
+                                  m=ff, k=d, x_row_stride=d, w_m_stride=d, w_k_stride=1, w_group_stride=ff * d, y_row_stride=ff,
+                                  tile_group=tg.data_ptr(), tile_row0=t0.data_ptr(), tile_rows=tr.data_ptr(), n_tiles=nt.data_ptr(),
+                                  max_tiles=max_tiles, x_row_index=pos_row.data_ptr(), y_row_index=pos_pair.data_ptr(),
+                                  max_tile_rows=rows, plain=plain))
+        outs.append(y.cpu())
+    ref = torch.einsum("pd,pfd->pf", x.double().repeat_interleave(top, 0), w.double()[expert.reshape(-1).long()])
+    assert (outs[0].double() - ref).abs().max() < 1e-4 and (outs[1].double() - ref).abs().max() < 1e-4
