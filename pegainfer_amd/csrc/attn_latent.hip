@@ -179,14 +179,18 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(float* __restric
 // One workgroup = 64 consecutive (token, head) rows of ONE request (4 waves x 16 rows) against key tiles of 32 cache entries,
 // v_mfma_f32_16x16x32_bf16 for both products:
 //   scores^T [32 keys x 16 rows]  = entries [32 x E] . q^T          A = entry rows from LDS, B = the wave's q rows (bf16 in LDS)
-//   out^T    [16 dims x 16 rows] += c^T [16 x 32 keys] . p^T        A = the latent tile TRANSPOSED in LDS, B = the lane's own p
+//   out^T    [16 dims x 16 rows] += c^T [16 x 32 keys] . p^T        A = the SAME row-major tile read transposed, B = the lane's own p
 // The score MFMA leaves lane (row l15, group g) with the scores of keys 4g..4g+3 and 16+4g..16+4g+3 of its row - exactly the
-// eight values the second product wants from that lane as its B operand, provided the reduction index is numbered
-// kidx = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4); the transposed latent tile is written in that numbering, so the
-// weights never move between lanes.  Every head of a token reads the same entries, so a tile of 64 rows (8 tokens x 8 heads,
-// or one decoded token's heads) shares each staged key tile.  Softmax state (max, sum) and the output accumulators are fp32;
-// q and the weights are rounded to bf16 where they enter the matrix cores.  Keys are split over blockIdx.y like the plain form.
+// eight values the second product wants from that lane as its B operand when the reduction index is numbered
+// kidx = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4): the weights never move between lanes.  The matching A fragment
+// (dim l15 of those eight keys) comes from two ds_read_b64_tr_b16: inside a 16-lane group lane 4j + c gives the address of
+// dims 4c..4c+3 of key row j, and lane i receives dim i of the four rows - so the latent tile is staged once, row-major, and
+// serves both products.  Every head of a token reads the same entries, so a tile of 64 rows (8 tokens x 8 heads, or one
+// decoded token's heads) shares each staged key tile.  The next key tile's global loads are issued into registers before the
+// current tile's products and written to LDS after them.  Softmax state (max, sum) and the output accumulators are fp32; q and
+// the weights are rounded to bf16 where they enter the matrix cores.  Keys are split over blockIdx.y like the plain form.
 constexpr int kTileRows = 64, kTileKeys = 32;
+constexpr int kLatPrefetch = 10;     // 16-byte chunks per thread and key tile: 32 keys x (E / 8) <= 2560 chunks, E <= 640
 
 template <int ND>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __restrict__ qc, float* __restrict__ o_lat,
@@ -201,11 +205,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
                                                                float scale, float* __restrict__ partial, int max_splits,
                                                                int split_keys) {
   extern __shared__ __align__(16) uint8_t lat_smem[];
+  typedef short v4s_t __attribute__((ext_vector_type(4)));
   const int E = r + dr, Epad = (E + 31) & ~31;
-  const int qs = Epad + 8, cs = Epad + 8, ts = kTileKeys + 8;      // LDS row strides (bf16 elements), 16-byte multiples
+  const int qs = Epad + 8, cs = Epad + 8;                          // LDS row strides (bf16 elements), 16-byte multiples
   uint16_t* Qs = reinterpret_cast<uint16_t*>(lat_smem);            // [64][qs]
   uint16_t* Ck = Qs + kTileRows * qs;                              // [32][cs]
-  uint16_t* Ct = Ck + kTileKeys * cs;                              // [ND * 16][ts]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l15 = lane & 15, g = lane >> 4;
   const int row0 = tile_row0[blockIdx.x], cnt = tile_rows[blockIdx.x], split = blockIdx.y;
   const int t_first = row0 / H, t_last = (row0 + cnt - 1) / H;
@@ -214,45 +218,74 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   if (j_lo > pmax) return;
   const int j_hi = min(pmax + 1, j_lo + split_keys);
   const int32_t* pages = page_ids + page_indptr[token_req[t_first]];
+  const int nchunk = E >> 3, tile_chunks = kTileKeys * nchunk;
+  u32x4 pre[kLatPrefetch];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < kLatPrefetch; ++i) {
+      const int c = tid + i * 256;
+      if (c < tile_chunks) {
+        const int kk = c / nchunk, ch = c - kk * nchunk;
+        const int j = min(j0 + kk, j_hi - 1);
+        pre[i] = *reinterpret_cast<const u32x4*>(latent_entry(cache, page_stride, layer_off, page_size, pages, j, E) + ch * 8);
+      }
+    }
+  };
+  fetch(j_lo);
   for (int i = tid; i < kTileRows * Epad; i += 256) {
     const int row = i / Epad, k = i - row * Epad;
     Qs[row * qs + k] = (row < cnt && k < E) ? f2bf(qc[(int64_t)(row0 + row) * E + k]) : (uint16_t)0;
   }
   for (int i = tid; i < kTileKeys * (Epad - E); i += 256) Ck[(i / (Epad - E)) * cs + E + i % (Epad - E)] = 0;
-  for (int i = tid; i < (ND * 16 - r) * kTileKeys; i += 256) Ct[(r + i / kTileKeys) * ts + i % kTileKeys] = 0;
   const int my_row = wave * 16 + l15;
   const int pq = my_row < cnt ? positions[(row0 + my_row) / H] : -1;
+  const bool wave_live = wave * 16 < cnt;                            // a wave without rows only helps staging
   f32x4 o[ND];
 #pragma unroll
   for (int d = 0; d < ND; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const int nchunk = E >> 3;
+  // per-lane element offset of the transposed reads inside the key tile: key row 4g + (l15 >> 2), dims 4 (l15 & 3) ..
+  const int tr_off = (4 * g + (l15 >> 2)) * cs + 4 * (l15 & 3);
   for (int j0 = j_lo; j0 < j_hi; j0 += kTileKeys) {
-    __syncthreads();
-    for (int c = tid; c < kTileKeys * nchunk; c += 256) {
-      const int kk = c / nchunk, ch = c - kk * nchunk;
-      const int j = min(j0 + kk, j_hi - 1);
-      const u32x4 v = *reinterpret_cast<const u32x4*>(latent_entry(cache, page_stride, layer_off, page_size, pages, j, E) + ch * 8);
-      *reinterpret_cast<u32x4*>(Ck + kk * cs + ch * 8) = v;
-      if (ch * 8 < r) {
-        const int kidx = kk < 16 ? 8 * (kk >> 2) + (kk & 3) : 8 * ((kk - 16) >> 2) + 4 + (kk & 3);
-        const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+    __syncthreads();                                                 // the previous tile's reads are done
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int d = ch * 8 + i;
-          if (d < r) Ct[d * ts + kidx] = (uint16_t)(i & 1 ? wv[i >> 1] >> 16 : wv[i >> 1] & 0xFFFFu);
-        }
+    for (int i = 0; i < kLatPrefetch; ++i) {
+      const int c = tid + i * 256;
+      if (c < tile_chunks) {
+        const int kk = c / nchunk, ch = c - kk * nchunk;
+        *reinterpret_cast<u32x4*>(Ck + kk * cs + ch * 8) = pre[i];
       }
     }
     __syncthreads();
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    for (int kb = 0; kb < Epad; kb += 32) {
-      const bf16x8_t qv = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Qs + my_row * qs + kb + g * 8));
-      const bf16x8_t k0 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ck + l15 * cs + kb + g * 8));
-      const bf16x8_t k1 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ck + (16 + l15) * cs + kb + g * 8));
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qv, s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qv, s1, 0, 0, 0);
+    if (j0 + kTileKeys < j_hi) fetch(j0 + kTileKeys);
+    if (!wave_live) continue;
+    // two independent accumulator pairs over alternating k slices: with one wave per SIMD the LDS read -> MFMA -> MFMA chain
+    // of a single pair would run at its latency
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f}, s3 = {0.f, 0.f, 0.f, 0.f};
+    const uint16_t* qp = Qs + my_row * qs + g * 8;
+    const uint16_t* kp0 = Ck + l15 * cs + g * 8;
+    const uint16_t* kp1 = Ck + (16 + l15) * cs + g * 8;
+    int kb = 0;
+#pragma unroll 2
+    for (; kb + 64 <= Epad; kb += 64) {
+      const bf16x8_t qa = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(qp + kb));
+      const bf16x8_t qb = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(qp + kb + 32));
+      const bf16x8_t a0 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp0 + kb));
+      const bf16x8_t a1 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp1 + kb));
+      const bf16x8_t b0 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp0 + kb + 32));
+      const bf16x8_t b1 = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp1 + kb + 32));
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qa, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qa, s1, 0, 0, 0);
+      s2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b0, qb, s2, 0, 0, 0);
+      s3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b1, qb, s3, 0, 0, 0);
     }
+    if (kb < Epad) {
+      const bf16x8_t qa = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(qp + kb));
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp0 + kb)), qa, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(kp1 + kb)), qa, s1, 0, 0, 0);
+    }
+    s0 += s2;
+    s1 += s3;
     float sc[8];
     float mx = -INFINITY;
 #pragma unroll
@@ -279,11 +312,16 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
     m = m_new;
     const u32x4 pw = {pack_bf2(ps[0], ps[1]), pack_bf2(ps[2], ps[3]), pack_bf2(ps[4], ps[5]), pack_bf2(ps[6], ps[7])};
     const bf16x8_t pv = __builtin_bit_cast(bf16x8_t, pw);
+    const __attribute__((address_space(3))) uint16_t* ck3 =
+        (const __attribute__((address_space(3))) uint16_t*)(Ck) + tr_off;
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       if (d * 16 >= r) break;
       o[d] *= corr;
-      const bf16x8_t cv = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(Ct + (d * 16 + l15) * ts + g * 8));
+      const v4s_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s_t __attribute__((address_space(3)))*)(ck3 + d * 16));
+      const v4s_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s_t __attribute__((address_space(3)))*)(ck3 + d * 16 + 16 * cs));
+      const u32x2 w0 = __builtin_bit_cast(u32x2, a0), w1 = __builtin_bit_cast(u32x2, a1);
+      const bf16x8_t cv = __builtin_bit_cast(bf16x8_t, u32x4{w0.x, w0.y, w1.x, w1.y});
       o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cv, pv, o[d], 0, 0, 0);
     }
   }
@@ -316,7 +354,7 @@ static void latent_attn_mfma_launch(const float* qc, float* o_lat, const uint16_
                                     const int32_t* tile_rows, int n_tiles, int H, int r, int dr, float scale, float* ws, int sp,
                                     int split_keys, hipStream_t s) {
   const int Epad = (r + dr + 31) & ~31;
-  const int lds = ((kTileRows + kTileKeys) * (Epad + 8) + ND * 16 * (kTileKeys + 8)) * 2;
+  const int lds = (kTileRows + kTileKeys) * (Epad + 8) * 2;
   auto kern = &latent_attn_mfma_kernel<ND>;
   static const bool once = (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                 160 * 1024), true);
@@ -364,9 +402,8 @@ int64_t pegainfer_latent_attention_workspace(int32_t n_tokens, int32_t heads, in
 
 int32_t pegainfer_latent_attention_tiled_ok(int32_t rank, int32_t rot, int64_t page_stride, int64_t layer_off, int32_t dtype) {
   const int Epad = (rank + rot + 31) & ~31;
-  const int nd = rank <= 64 ? 4 : rank <= 128 ? 8 : rank <= 256 ? 16 : 32;
   return dtype == kDtBf16 && rank % 16 == 0 && rank <= 512 && rot % 8 == 0 && page_stride % 8 == 0 && layer_off % 8 == 0 &&
-         ((kTileRows + kTileKeys) * (Epad + 8) + nd * 16 * (kTileKeys + 8)) * 2 <= 160 * 1024;
+         kTileKeys * ((rank + rot) / 8) <= kLatPrefetch * 256 && (kTileRows + kTileKeys) * (Epad + 8) * 2 <= 160 * 1024;
 }
 
 pegainfer_status_t pegainfer_latent_attention(const float* qc, float* o_lat, const void* cache, int64_t page_stride,
