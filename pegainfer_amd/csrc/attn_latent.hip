@@ -160,18 +160,26 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const float* __restric
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(float* __restrict__ o_lat, const float* __restrict__ partial,
                                                                 const int32_t* __restrict__ positions, int H, int r,
                                                                 int max_splits, int split_keys) {
+  extern __shared__ float wsm[];   // [n_splits] weights exp(m_s - m) / l
+  __shared__ float red[4];
   const int t = blockIdx.x, h = blockIdx.y;
   const int n_splits = (positions[t] + split_keys) / split_keys;
   if (n_splits <= 1) return;
   const float* part = partial + ((int64_t)t * H + h) * max_splits * (r + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part[(int64_t)s * (r + 2)]);
+  // the splits' maxima and sums are read in parallel (one thread each), combined in split order
+  float mloc = -INFINITY;
+  for (int s = threadIdx.x; s < n_splits; s += 256) mloc = fmaxf(mloc, part[(int64_t)s * (r + 2)]);
+  const float m = block_max256(mloc, red);
+  for (int s = threadIdx.x; s < n_splits; s += 256) wsm[s] = expf(part[(int64_t)s * (r + 2)] - m);
+  __syncthreads();
   float l = 0.f;
-  for (int s = 0; s < n_splits; ++s) l += part[(int64_t)s * (r + 2) + 1] * expf(part[(int64_t)s * (r + 2)] - m);
+  for (int s = 0; s < n_splits; ++s) l += part[(int64_t)s * (r + 2) + 1] * wsm[s];
+  const float inv = 1.0f / l;
   for (int d = threadIdx.x; d < r; d += 256) {
     float a = 0.f;
-    for (int s = 0; s < n_splits; ++s) a += part[(int64_t)s * (r + 2) + 2 + d] * expf(part[(int64_t)s * (r + 2)] - m);
-    o_lat[((int64_t)t * H + h) * r + d] = a / l;
+#pragma unroll 4
+    for (int s = 0; s < n_splits; ++s) a = fmaf(part[(int64_t)s * (r + 2) + 2 + d], wsm[s], a);
+    o_lat[((int64_t)t * H + h) * r + d] = a * inv;
   }
 }
 
@@ -219,22 +227,42 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   const int j_hi = min(pmax + 1, j_lo + split_keys);
   const int32_t* pages = page_ids + page_indptr[token_req[t_first]];
   const int nchunk = E >> 3, tile_chunks = kTileKeys * nchunk;
+  // this thread's chunks of a key tile: key kk, element offset ch * 8 - fixed for the whole loop, so the integer divisions
+  // happen once (a wave64 VALU instruction costs four cycles; an emulated division about forty of them)
   u32x4 pre[kLatPrefetch];
+  int ck_kk[kLatPrefetch], ck_el[kLatPrefetch];
+#pragma unroll
+  for (int i = 0; i < kLatPrefetch; ++i) {
+    const int c = tid + i * 256;
+    const int kk = c < tile_chunks ? c / nchunk : -1;
+    ck_kk[i] = kk;
+    ck_el[i] = kk < 0 ? 0 : (c - kk * nchunk) * 8;
+  }
+  const int pshift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
   auto fetch = [&](int j0) {
 #pragma unroll
     for (int i = 0; i < kLatPrefetch; ++i) {
-      const int c = tid + i * 256;
-      if (c < tile_chunks) {
-        const int kk = c / nchunk, ch = c - kk * nchunk;
-        const int j = min(j0 + kk, j_hi - 1);
-        pre[i] = *reinterpret_cast<const u32x4*>(latent_entry(cache, page_stride, layer_off, page_size, pages, j, E) + ch * 8);
+      if (ck_kk[i] >= 0) {
+        const int j = min(j0 + ck_kk[i], j_hi - 1);
+        const int pg = pshift >= 0 ? j >> pshift : j / page_size;
+        const int slot = pshift >= 0 ? j & (page_size - 1) : j - pg * page_size;
+        pre[i] = *reinterpret_cast<const u32x4*>(cache + (int64_t)pages[pg] * page_stride + layer_off + (int64_t)slot * E + ck_el[i]);
       }
     }
   };
   fetch(j_lo);
-  for (int i = tid; i < kTileRows * Epad; i += 256) {
-    const int row = i / Epad, k = i - row * Epad;
-    Qs[row * qs + k] = (row < cnt && k < E) ? f2bf(qc[(int64_t)(row0 + row) * E + k]) : (uint16_t)0;
+  {  // q rows -> bf16 in LDS, eight values per step; only the 16-row blocks that hold rows are staged
+    const int qchunks = Epad >> 3, rows_staged = min(kTileRows, (cnt + 15) & ~15);
+    for (int c = tid; c < rows_staged * qchunks; c += 256) {
+      const int row = c / qchunks, k = (c - row * qchunks) * 8;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row < cnt && k < E) {
+        const float* src = qc + (int64_t)(row0 + row) * E + k;
+        const f32x4 a = *reinterpret_cast<const f32x4*>(src), b = *reinterpret_cast<const f32x4*>(src + 4);
+        v = u32x4{pack_bf2(a.x, a.y), pack_bf2(a.z, a.w), pack_bf2(b.x, b.y), pack_bf2(b.z, b.w)};
+      }
+      *reinterpret_cast<u32x4*>(Qs + row * qs + k) = v;
+    }
   }
   for (int i = tid; i < kTileKeys * (Epad - E); i += 256) Ck[(i / (Epad - E)) * cs + E + i % (Epad - E)] = 0;
   const int my_row = wave * 16 + l15;
@@ -249,13 +277,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   for (int j0 = j_lo; j0 < j_hi; j0 += kTileKeys) {
     __syncthreads();                                                 // the previous tile's reads are done
 #pragma unroll
-    for (int i = 0; i < kLatPrefetch; ++i) {
-      const int c = tid + i * 256;
-      if (c < tile_chunks) {
-        const int kk = c / nchunk, ch = c - kk * nchunk;
-        *reinterpret_cast<u32x4*>(Ck + kk * cs + ch * 8) = pre[i];
-      }
-    }
+    for (int i = 0; i < kLatPrefetch; ++i)
+      if (ck_kk[i] >= 0) *reinterpret_cast<u32x4*>(Ck + ck_kk[i] * cs + ck_el[i]) = pre[i];
     __syncthreads();
     if (j0 + kTileKeys < j_hi) fetch(j0 + kTileKeys);
     if (!wave_live) continue;
@@ -299,11 +322,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
     const float m_new = fmaxf(m, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = expf(m - m_use);
+    const float corr = __expf(m - m_use);
     float ps[8], lsum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      ps[i] = bf16_round_f(expf(sc[i] - m_use));     // the sum uses the weights as the matrix core sees them
+      ps[i] = bf16_round_f(__expf(sc[i] - m_use));   // the sum uses the weights as the matrix core sees them
       lsum += ps[i];
     }
     lsum += __shfl_xor(lsum, 16, kWave);
@@ -314,10 +337,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
     const bf16x8_t pv = __builtin_bit_cast(bf16x8_t, pw);
     const __attribute__((address_space(3))) uint16_t* ck3 =
         (const __attribute__((address_space(3))) uint16_t*)(Ck) + tr_off;
+    // the running maximum of most rows stops moving after the first tiles: rescale only when some row of the wave needs it
+    if (__any(corr != 1.0f)) {
+#pragma unroll
+      for (int d = 0; d < ND; ++d) o[d] *= corr;
+    }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       if (d * 16 >= r) break;
-      o[d] *= corr;
       const v4s_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s_t __attribute__((address_space(3)))*)(ck3 + d * 16));
       const v4s_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s_t __attribute__((address_space(3)))*)(ck3 + d * 16 + 16 * cs));
       const u32x2 w0 = __builtin_bit_cast(u32x2, a0), w1 = __builtin_bit_cast(u32x2, a1);
@@ -442,7 +469,7 @@ pegainfer_status_t pegainfer_latent_attention(const float* qc, float* o_lat, con
         }))
       return (pegainfer_status_t)hipErrorInvalidValue;
   }
-  if (sp > 1) latent_attn_merge_kernel<<<dim3(n_tokens, heads), 256, 0, s>>>(o_lat, workspace, positions, heads, rank, sp, sk);
+  if (sp > 1) latent_attn_merge_kernel<<<dim3(n_tokens, heads), 256, (size_t)sp * sizeof(float), s>>>(o_lat, workspace, positions, heads, rank, sp, sk);
   return (pegainfer_status_t)hipGetLastError();
 }
 

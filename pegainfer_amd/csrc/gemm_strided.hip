@@ -227,37 +227,53 @@ __global__ __launch_bounds__(256) void gemm_strided_rows_kernel(pegainfer_gemm_d
   __syncthreads();
   TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
   const int m_base = blockIdx.y * kRowsFormOutputs;
-  for (int mi = wave; mi < kRowsFormOutputs; mi += 4) {
-    const int m = m_base + mi;
-    if (m >= d.m) break;
-    const TW* wrow = W + (int64_t)m * d.w_m_stride;
-    float acc[R];
+  // a wave owns 8 of the workgroup's 32 outputs and walks them four at a time: four independent weight streams in flight
+  constexpr int MB = 4;
+  for (int mg = 0; mg < kRowsFormOutputs / 4; mg += MB) {
+    const int mw = m_base + wave * (kRowsFormOutputs / 4) + mg;
+    if (mw >= d.m) break;
+    float acc[MB][R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
-#pragma unroll 2
+    for (int q = 0; q < MB; ++q)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[q][r] = 0.f;
     for (int k = lane * 8; k < K; k += 512) {
-      float wv[8];
-      Vec8<TW>::load(wrow + k, wv);
+      float wv[MB][8];
+#pragma unroll
+      for (int q = 0; q < MB; ++q) {
+        const int m = min(mw + q, d.m - 1);          // a clamped row is loaded and dropped at the store
+        Vec8<TW>::load(W + (int64_t)m * d.w_m_stride + k, wv[q]);
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const f32x4 xa = *reinterpret_cast<const f32x4*>(xr + r * K + k), xb = *reinterpret_cast<const f32x4*>(xr + r * K + k + 4);
-        float a = acc[r];
-        a = fmaf(wv[0], xa.x, a); a = fmaf(wv[1], xa.y, a); a = fmaf(wv[2], xa.z, a); a = fmaf(wv[3], xa.w, a);
-        a = fmaf(wv[4], xb.x, a); a = fmaf(wv[5], xb.y, a); a = fmaf(wv[6], xb.z, a); a = fmaf(wv[7], xb.w, a);
-        acc[r] = a;
+#pragma unroll
+        for (int q = 0; q < MB; ++q) {
+          float a = acc[q][r];
+          a = fmaf(wv[q][0], xa.x, a); a = fmaf(wv[q][1], xa.y, a); a = fmaf(wv[q][2], xa.z, a); a = fmaf(wv[q][3], xa.w, a);
+          a = fmaf(wv[q][4], xb.x, a); a = fmaf(wv[q][5], xb.y, a); a = fmaf(wv[q][6], xb.z, a); a = fmaf(wv[q][7], xb.w, a);
+          acc[q][r] = a;
+        }
       }
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    for (int q = 0; q < MB; ++q)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[q][r] = wave_sum(acc[q][r]);
     if (lane == 0) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (yrow[r] < 0) continue;
-        float v = acc[r];
-        if (d.epilogue == PEGAINFER_EPI_RELU_SQ) { v = fmaxf(v, 0.f); v *= v; }
-        else if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
-          v *= sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
-        st(Y + (int64_t)yrow[r] * d.y_row_stride + m, v);
+      for (int q = 0; q < MB; ++q) {
+        const int m = mw + q;
+        if (m >= d.m) break;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          if (yrow[r] < 0) continue;
+          float v = acc[q][r];
+          if (d.epilogue == PEGAINFER_EPI_RELU_SQ) { v = fmaxf(v, 0.f); v *= v; }
+          else if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
+            v *= sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
+          st(Y + (int64_t)yrow[r] * d.y_row_stride + m, v);
+        }
       }
     }
   }

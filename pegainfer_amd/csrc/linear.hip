@@ -978,8 +978,14 @@ static pegainfer_status_t gemv_fused_impl(const Half* W, const Half* X, Half* Y,
   if ((flags & ~kGemvRoundSum) != 0 && (T > 4 || t1_uses_mfma())) return (pegainfer_status_t)hipErrorInvalidValue;
   if (flags == kGemvRoundSum && T > 4 && (T > 16 || (K & 63) != 0)) return (pegainfer_status_t)hipErrorInvalidValue;
   GemvFusedArgs a{W, X, Y, M, T, K, residual, norm_weight, hidden_out, eps, silu_intermediate, 0, flags};
-  const bool ok = silu_intermediate > 0 ? decode_gemm_dispatch<kEpiSilu>(a, as_stream(stream))
-                                        : decode_gemm_dispatch<kEpiStore>(a, as_stream(stream));
+  bool ok = silu_intermediate > 0 ? decode_gemm_dispatch<kEpiSilu>(a, as_stream(stream))
+                                  : decode_gemm_dispatch<kEpiStore>(a, as_stream(stream));
+  if (!ok && !norm_weight && !residual && silu_intermediate == 0 && flags == 0 && (K & 63) == 0) {
+    // the plain form of a shape this entry has always accepted but the skinny kernel cannot take (above 8 columns with
+    // K % 128 == 64): the tiled / naive routes of gemm_cuda
+    gemm_dispatch(W, X, Y, M, T, K, as_stream(stream));
+    ok = true;
+  }
   return ok ? (pegainfer_status_t)hipGetLastError() : (pegainfer_status_t)hipErrorInvalidValue;
 }
 

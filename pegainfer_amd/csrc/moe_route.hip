@@ -26,26 +26,38 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const A* x = h + (size_t)row * d;
   const bool vec = (d & 7) == 0 && aligned16(x) && aligned16(wr);
-  for (int e = wave; e < E; e += 4) {
-    const A* w = wr + (size_t)e * d;
-    float a = 0.f;
+  // a wave takes four experts at a time (four independent weight streams in flight), waves interleaved over the groups of four
+  constexpr int EB = 4;
+  for (int e0 = wave * EB; e0 < E; e0 += 4 * EB) {
+    float a[EB] = {0.f, 0.f, 0.f, 0.f};
     if (vec) {
-#pragma unroll 2
       for (int i = lane * 8; i < d; i += 512) {
-        float xv[8], wv[8];
+        float xv[8];
         Vec8<A>::load(x + i, xv);
-        Vec8<A>::load(w + i, wv);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) a = fmaf(xv[k], wv[k], a);
+        for (int q = 0; q < EB; ++q) {
+          float wv[8];
+          Vec8<A>::load(wr + (size_t)min(e0 + q, E - 1) * d + i, wv);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) a[q] = fmaf(xv[k], wv[k], a[q]);
+        }
       }
     } else {
-      for (int i = lane; i < d; i += 64) a = fmaf(ld(x + i), ld(w + i), a);
+      for (int i = lane; i < d; i += 64) {
+        const float xv = ld(x + i);
+#pragma unroll
+        for (int q = 0; q < EB; ++q) a[q] = fmaf(xv, ld(wr + (size_t)min(e0 + q, E - 1) * d + i), a[q]);
+      }
     }
-    a = wave_sum(a);
-    if (lane == 0) {
-      const float sc = sigmoid_f(a);
-      s[e] = sc;
-      ch[e] = corr ? sc + ld(corr + e) : sc;
+#pragma unroll
+    for (int q = 0; q < EB; ++q) {
+      const float z = wave_sum(a[q]);
+      const int e = e0 + q;
+      if (lane == 0 && e < E) {
+        const float sc = sigmoid_f(z);
+        s[e] = sc;
+        ch[e] = corr ? sc + ld(corr + e) : sc;
+      }
     }
   }
   __syncthreads();

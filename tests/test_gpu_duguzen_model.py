@@ -240,3 +240,26 @@ def test_greedy_generation_through_the_scheduler(dtype):
     assert eng.available_pages() == eng.capacity_pages()          # finished requests gave their pages back
     sch.close()
     eng.close()
+
+
+def test_command_line_generates_like_the_plain_restatement(tmp_path):
+    import subprocess
+    import sys
+    from safetensors.torch import save_file
+    cfg = C.config_tiny()
+    w = C.random_weights(cfg, 19)
+    json.dump(cfg, open(tmp_path / "config.json", "w"))
+    save_file({k: v.bfloat16().contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    prompt = C.tokens_for(cfg, 11, 6)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-m", "pegainfer_amd", "generate", "--model", str(tmp_path), "--dtype", "float32",
+                        "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5"], cwd=root, capture_output=True,
+                       text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    got = json.loads([l for l in p.stdout.split("\n") if l.startswith("{")][-1])["tokens"]
+    seq = list(prompt)
+    for tok in got:
+        lg = C.oracle_logits(cfg, w, seq)[-1]
+        assert tok == int(lg.argmax()) or lg[tok] >= lg.max() - 1e-3
+        seq.append(tok)
+    assert len(got) == 5
