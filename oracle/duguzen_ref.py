@@ -32,8 +32,12 @@ def read_config(path):
 
 def owner(cfg, i):
     """index of the layer whose tensors layer i computes with"""
-    j = cfg["layers"][i].get("weights_of")
-    return i if j is None else int(j)
+    for _ in range(len(cfg["layers"])):
+        j = cfg["layers"][i].get("weights_of")
+        if j is None or int(j) == i:
+            return i
+        i = int(j)
+    raise ValueError("weights_of forms a cycle")
 
 
 def dyt(x, w, name):

@@ -211,8 +211,12 @@ struct Model {
       off += (int64_t)kPageSize * c.entry();
       layers.push_back(c);
     }
-    for (auto& c : layers)
-      if (layers[c.owner].owner != c.owner) return set_error("config: weights_of names a layer without tensors of its own");
+    for (auto& c : layers) {   // a borrowed layer may itself borrow: follow the chain to the layer that owns tensors
+      int o = c.owner, hops = 0;
+      while (layers[o].owner != o && hops++ < (int)layers.size()) o = layers[o].owner;
+      if (layers[o].owner != o) return set_error("config: weights_of forms a cycle");
+      c.owner = o;
+    }
     page_stride = off;
     weights.resize(layers.size());
     for (auto& c : layers) {

@@ -80,3 +80,18 @@ def test_sigmoid_gate_and_squared_relu():
     a = R.latent_attention(h, w, "l0.mix", cfg["layers"][0]["mixer"], 1e-5, pos)
     b = R.latent_attention(h, w_closed, "l0.mix", cfg["layers"][0]["mixer"], 1e-5, pos)
     assert not torch.allclose(a, 2 * b) and torch.isfinite(a).all()      # gate 0.5 everywhere is one particular scaling
+
+
+def test_borrowing_from_a_layer_that_borrows():
+    cfg = C.config_a()
+    w = C.random_weights(cfg, 6)
+    toks = C.tokens_for(cfg, 9, 1)
+    ref = C.oracle_logits(cfg, w, toks)
+    chained = {**cfg, "layers": [dict(l) for l in cfg["layers"]]}
+    chained["layers"][4]["weights_of"] = 1          # as before
+    chained["layers"][2]["weights_of"] = 0
+    chained["layers"].append({**cfg["layers"][2], "weights_of": 2})     # layer 5 borrows from 2, which borrows from 0
+    direct = {**cfg, "layers": cfg["layers"] + [{**cfg["layers"][2], "weights_of": 0}]}
+    assert R.owner(chained, 5) == 0
+    assert np.allclose(C.oracle_logits(chained, w, toks), C.oracle_logits(direct, w, toks), atol=1e-12)
+    assert not np.allclose(C.oracle_logits(direct, w, toks), ref, atol=1e-6)

@@ -263,3 +263,17 @@ def test_command_line_generates_like_the_plain_restatement(tmp_path):
         assert tok == int(lg.argmax()) or lg[tok] >= lg.max() - 1e-3
         seq.append(tok)
     assert len(got) == 5
+
+
+def test_a_layer_that_borrows_from_a_borrowing_layer():
+    cfg = C.config_a()
+    cfg["layers"].append({**cfg["layers"][2], "weights_of": 2})      # layer 5 -> layer 2 -> layer 0, with a cache of its own
+    w = C.random_weights(cfg, 21)
+    toks = C.tokens_for(cfg, 40, 7)
+    ref = C.oracle_logits(cfg, w, toks)
+    eng = C.engine_for(cfg, w, "float32")
+    assert eng.layer_runs == 6
+    r = eng.new_request()
+    got = np.concatenate([eng.step([(r, toks[:33])], want=list(range(33))), eng.step([(r, toks[33:])], want=list(range(7)))])
+    check(got, ref, "float32")
+    eng.close()
