@@ -45,7 +45,7 @@ pegainfer_status_t pegainfer_silu_mul_rows(const void* gate_up, void* out, int32
 
 /* ---- strided / batched / grouped GEMM:  y[row, g, m] = sum_k x[row, g, k] * w[g, m, k]  (+ epilogue) ----
  * Dense form (tile_group == NULL): `rows` rows in each of `groups` groups.
- * Grouped form: a device-side table of row tiles, each of <= 64 consecutive POSITIONS of a sorted list that belong to
+ * Grouped form: a device-side table of row tiles, each of <= 64 (or 128: tile_rows_cap) consecutive POSITIONS of a sorted list that belong to
  * one group (expert); positions map to x / y rows through x_row_index / y_row_index (NULL = identity).  Tiles beyond
  * *n_tiles exit; the grid is max_tiles wide.
  * Three kernels behind one entry: an fp32-FMA tile kernel (any sizes and strides, both storage types), a matrix-core tile
@@ -73,7 +73,8 @@ typedef struct {
   const void* gate;
   int32_t gate_dtype;
   int64_t gate_row_stride;
-  int32_t max_tile_rows;     /* grouped form: an upper bound of tile_rows the caller knows (0 = 64) */
+  int32_t max_tile_rows;     /* grouped form: an upper bound of tile_rows the caller knows (0 = tile_rows_cap) */
+  int32_t tile_rows_cap;     /* grouped form: the rows_per_tile the table was cut with (0 = 64) */
   int32_t plain;             /* != 0: always the fp32-FMA tile kernel (exact products of the stored values) */
 } pegainfer_gemm_desc;
 pegainfer_status_t pegainfer_gemm_strided(const pegainfer_gemm_desc* d, pegainfer_stream_t stream);
@@ -126,13 +127,14 @@ pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_
                                                    int32_t* out_expert, float* out_weight, int32_t d, int32_t experts,
                                                    int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
                                                    int32_t dtype, pegainfer_stream_t stream);
-/* Sort the rows * top (row, choice) pairs by expert into a position list and cut it into row tiles of <= 64 positions:
+/* Sort the rows * top (row, choice) pairs by expert into a position list and cut it into row tiles of <= rows_per_tile
+ * (64 or 128) positions:
  *   pos_pair[p] = pair index (row * top + choice) at position p;  pos_row[p] = its row
- *   tile_group / tile_row0 / tile_rows [max_tiles], *n_tiles;  max_tiles >= ceil(pairs / 64) + experts
+ *   tile_group / tile_row0 / tile_rows [max_tiles], *n_tiles;  max_tiles >= ceil(pairs / rows_per_tile) + experts
  * One workgroup, counters in LDS (experts <= 8192).  The order inside an expert is arbitrary; results do not depend on it. */
 pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, int32_t top, int32_t experts,
                                         int32_t* pos_pair, int32_t* pos_row, int32_t* tile_group, int32_t* tile_row0,
-                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles,
+                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles, int32_t rows_per_tile,
                                         pegainfer_stream_t stream);
 /* out[row, :] = sum_c weight[row, c] * y_pairs[row * top + c, :]   (c ascending; y_pairs fp32) */
 pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,

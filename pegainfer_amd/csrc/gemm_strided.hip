@@ -97,8 +97,8 @@ __global__ __launch_bounds__(256) void gemm_strided_kernel(pegainfer_gemm_desc d
 
 
 // ------------------------------------------------------------------ matrix-core form (bf16 weights, k contiguous)
-// Same 64 x 64 tile and the same addressing (groups, gathered rows, tile table), K in slices of 64 staged as bf16, four waves
-// in a 2 x 2 arrangement, each 2 x 2 blocks of v_mfma_f32_16x16x32_bf16.  fp32 x (the attention output in front of the value
+// The same addressing (groups, gathered rows, tile table), K in slices of 64 staged as bf16 through registers (the next slice
+// is in flight while this one is multiplied), four waves in a 2 x 2 arrangement of v_mfma_f32_16x16x32_bf16 blocks.  fp32 x (the attention output in front of the value
 // up-projection) is rounded to bf16 while it is staged.  Needs 16-byte chunks: K % 8 == 0, strides % 8 == 0, aligned bases.
 constexpr int MK = 64, MS = MK + 8;
 
@@ -108,25 +108,29 @@ __device__ __forceinline__ u32x4 stage8(const float* p) {
   return u32x4{pack_bf2(a.x, a.y), pack_bf2(a.z, a.w), pack_bf2(b.x, b.y), pack_bf2(b.z, b.w)};
 }
 
-template <typename TX, typename TY, typename TG>
+// Output tile TR rows x 128 outputs (TR = 64 or 128): with 64 x 64 tiles the kernel moved 32 flop per byte staged and sat on
+// the L2 -> CU bandwidth (7.5 TB/s of staging traffic at 1024 tokens x 4 experts); 128 x 128 halves the bytes per flop.
+constexpr int MM = 128;
+
+template <typename TX, typename TY, typename TG, int TR>
 __global__ __launch_bounds__(256) void gemm_strided_mfma_kernel(pegainfer_gemm_desc d) {
-  __shared__ __align__(16) uint16_t xs[GT * MS];
-  __shared__ __align__(16) uint16_t ws[GM * MS];
-  __shared__ int xrow[GT], yrow[GT];
+  __shared__ __align__(16) uint16_t xs[TR * MS];
+  __shared__ __align__(16) uint16_t ws[MM * MS];
+  __shared__ int xrow[TR], yrow[TR];
   int g, row0, nrows;
   if (d.tile_group) {
     if ((int)blockIdx.x >= *d.n_tiles) return;
     g = d.tile_group[blockIdx.x];
     row0 = d.tile_row0[blockIdx.x];
-    nrows = d.tile_rows[blockIdx.x];
+    nrows = min(TR, d.tile_rows[blockIdx.x]);
   } else {
     g = blockIdx.z;
-    row0 = blockIdx.x * GT;
-    nrows = min(GT, d.rows - row0);
+    row0 = blockIdx.x * TR;
+    nrows = min(TR, d.rows - row0);
   }
-  const int m0 = blockIdx.y * GM;
+  const int m0 = blockIdx.y * MM;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l15 = lane & 15, gq = lane >> 4;
-  if (tid < GT) {
+  if (tid < TR) {
     const int p = row0 + tid;
     xrow[tid] = tid < nrows ? (d.x_row_index ? d.x_row_index[p] : p) : -1;
     yrow[tid] = tid < nrows ? (d.y_row_index ? d.y_row_index[p] : p) : -1;
@@ -134,41 +138,62 @@ __global__ __launch_bounds__(256) void gemm_strided_mfma_kernel(pegainfer_gemm_d
   __syncthreads();
   const TX* X = static_cast<const TX*>(d.x) + (int64_t)g * d.x_group_stride;
   const uint16_t* W = static_cast<const uint16_t*>(d.w) + (int64_t)g * d.w_group_stride;
-  const int wr = (wave & 1) * 32, wm = (wave >> 1) * 32;
-  f32x4 acc[2][2];
+  constexpr int RJ = TR / 32;                       // 16-row blocks per wave
+  const int wr = (wave & 1) * (TR / 2), wm = (wave >> 1) * 64;
+  f32x4 acc[4][RJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < RJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  for (int k0 = 0; k0 < d.k; k0 += MK) {
+  constexpr int XC = TR * (MK / 8) / 256, WC = MM * (MK / 8) / 256;   // chunks per thread and K slice
+  // this thread's rows are the same in every K slice: resolve them once
+  const TX* xsrc[XC];
+  const uint16_t* wsrc[WC];
 #pragma unroll
-    for (int c = tid; c < GT * (MK / 8); c += 256) {
-      const int r = c >> 3, kk = k0 + (c & 7) * 8;
-      const int src = xrow[r];
-      *reinterpret_cast<u32x4*>(xs + r * MS + (c & 7) * 8) = (src >= 0 && kk < d.k) ? stage8(X + (int64_t)src * d.x_row_stride + kk) : zero;
-      *reinterpret_cast<u32x4*>(ws + r * MS + (c & 7) * 8) =
-          (m0 + r < d.m && kk < d.k) ? stage8(W + (int64_t)(m0 + r) * d.w_m_stride + kk) : zero;
-    }
+  for (int i = 0; i < XC; ++i) {
+    const int c = tid + i * 256, src = xrow[c >> 3];
+    xsrc[i] = src >= 0 ? X + (int64_t)src * d.x_row_stride + (c & 7) * 8 : nullptr;
+  }
+#pragma unroll
+  for (int i = 0; i < WC; ++i) {
+    const int c = tid + i * 256, m = m0 + (c >> 3);
+    wsrc[i] = m < d.m ? W + (int64_t)m * d.w_m_stride + (c & 7) * 8 : nullptr;
+  }
+  u32x4 px[XC], pw[WC];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < XC; ++i) px[i] = (xsrc[i] && k0 + ((tid + i * 256) & 7) * 8 < d.k) ? stage8(xsrc[i] + k0) : zero;
+#pragma unroll
+    for (int i = 0; i < WC; ++i) pw[i] = (wsrc[i] && k0 + ((tid + i * 256) & 7) * 8 < d.k) ? stage8(wsrc[i] + k0) : zero;
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < d.k; k0 += MK) {
     __syncthreads();
+#pragma unroll
+    for (int i = 0; i < XC; ++i) { const int c = tid + i * 256; *reinterpret_cast<u32x4*>(xs + (c >> 3) * MS + (c & 7) * 8) = px[i]; }
+#pragma unroll
+    for (int i = 0; i < WC; ++i) { const int c = tid + i * 256; *reinterpret_cast<u32x4*>(ws + (c >> 3) * MS + (c & 7) * 8) = pw[i]; }
+    __syncthreads();
+    if (k0 + MK < d.k) fetch(k0 + MK);            // the next slice's loads fly while this one is multiplied
 #pragma unroll
     for (int ks = 0; ks < MK; ks += 32) {
-      bf16x8_t a[2], b[2];
+      bf16x8_t a[4], b[RJ];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < 4; ++i)
         a[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(ws + (wm + i * 16 + l15) * MS + ks + gq * 8));
-        b[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xs + (wr + i * 16 + l15) * MS + ks + gq * 8));
-      }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int j = 0; j < RJ; ++j)
+        b[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xs + (wr + j * 16 + l15) * MS + ks + gq * 8));
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < RJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    __syncthreads();
   }
   TY* Y = static_cast<TY*>(d.y) + (int64_t)g * d.y_group_stride;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < RJ; ++j) {
     const int r = wr + j * 16 + l15;
     const int dst = yrow[r];
     if (dst < 0) continue;
@@ -176,7 +201,7 @@ __global__ __launch_bounds__(256) void gemm_strided_mfma_kernel(pegainfer_gemm_d
     if (d.epilogue == PEGAINFER_EPI_SIGMOID_GATE)
       scale = sigmoid_f(ld(static_cast<const TG*>(d.gate) + (int64_t)xrow[r] * d.gate_row_stride + g));
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int m = m0 + wm + i * 16 + gq * 4 + e;
@@ -187,6 +212,15 @@ __global__ __launch_bounds__(256) void gemm_strided_mfma_kernel(pegainfer_gemm_d
         st(Y + (int64_t)dst * d.y_row_stride + m, v);
       }
   }
+}
+
+template <typename TX, typename TY, typename TG>
+static void mfma_form_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
+  const bool big = d.tile_group ? d.tile_rows_cap >= 128 : d.rows > 64;
+  const int TR = big ? 128 : 64;
+  dim3 grid(d.tile_group ? d.max_tiles : ceil_div(d.rows, TR), ceil_div(d.m, MM), d.tile_group ? 1 : d.groups);
+  if (big) gemm_strided_mfma_kernel<TX, TY, TG, 128><<<grid, 256, 0, s>>>(d);
+  else gemm_strided_mfma_kernel<TX, TY, TG, 64><<<grid, 256, 0, s>>>(d);
 }
 
 // ------------------------------------------------------------------ few-rows form (decode)
@@ -297,26 +331,28 @@ static inline bool chunks_ok(const pegainfer_gemm_desc& d) {
 }
 
 template <typename TX, typename TW, typename TY>
-static void gemm_strided_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
+static bool gemm_strided_launch(const pegainfer_gemm_desc& d, hipStream_t s) {
   dim3 grid(d.tile_group ? d.max_tiles : ceil_div(d.rows, GT), ceil_div(d.m, GM), d.tile_group ? 1 : d.groups);
   const bool gate32 = d.gate_dtype == kDtF32;
   if (!d.plain && chunks_ok(d)) {
     // few rows per tile: stream the weights once (both storage types, fp32 arithmetic)
-    const int tr = d.tile_group ? (d.max_tile_rows > 0 ? d.max_tile_rows : GT) : d.rows;
+    const int tr = d.tile_group ? (d.max_tile_rows > 0 ? d.max_tile_rows : (d.tile_rows_cap > 0 ? d.tile_rows_cap : GT)) : d.rows;
     const int R = tr <= 1 ? 1 : tr <= 4 ? 4 : tr <= 8 ? 8 : 0;
     if (R && (size_t)R * d.k * sizeof(float) <= 150 * 1024) {
       if (gate32) { if (R == 1) rows_form_launch<TX, TW, TY, float, 1>(d, s); else if (R == 4) rows_form_launch<TX, TW, TY, float, 4>(d, s); else rows_form_launch<TX, TW, TY, float, 8>(d, s); }
       else { if (R == 1) rows_form_launch<TX, TW, TY, uint16_t, 1>(d, s); else if (R == 4) rows_form_launch<TX, TW, TY, uint16_t, 4>(d, s); else rows_form_launch<TX, TW, TY, uint16_t, 8>(d, s); }
-      return;
+      return true;
     }
     if constexpr (std::is_same<TW, uint16_t>::value) {   // bf16 weights: the matrix cores
-      if (gate32) gemm_strided_mfma_kernel<TX, TY, float><<<grid, 256, 0, s>>>(d);
-      else gemm_strided_mfma_kernel<TX, TY, uint16_t><<<grid, 256, 0, s>>>(d);
-      return;
+      if (gate32) mfma_form_launch<TX, TY, float>(d, s);
+      else mfma_form_launch<TX, TY, uint16_t>(d, s);
+      return true;
     }
   }
+  if (d.tile_group && d.tile_rows_cap > GT) return false;   // a table cut for 128-row tiles cannot be walked by the 64-row form
   if (gate32) gemm_strided_kernel<TX, TW, TY, float><<<grid, 256, 0, s>>>(d);
   else gemm_strided_kernel<TX, TW, TY, uint16_t><<<grid, 256, 0, s>>>(d);
+  return true;
 }
 
 }  // namespace pk
@@ -328,13 +364,15 @@ extern "C" pegainfer_status_t pegainfer_gemm_strided(const pegainfer_gemm_desc* 
   if (d.tile_group ? d.max_tiles <= 0 : (d.rows <= 0 || d.groups <= 0)) return 0;
   hipStream_t s = as_stream(stream);
   const int key = (d.x_dtype << 2) | (d.w_dtype << 1) | d.y_dtype;
+  bool ok = false;
   switch (key) {
-    case 0: gemm_strided_launch<uint16_t, uint16_t, uint16_t>(d, s); break;
-    case 1: gemm_strided_launch<uint16_t, uint16_t, float>(d, s); break;
-    case 4: gemm_strided_launch<float, uint16_t, uint16_t>(d, s); break;
-    case 5: gemm_strided_launch<float, uint16_t, float>(d, s); break;
-    case 7: gemm_strided_launch<float, float, float>(d, s); break;
-    default: return (pegainfer_status_t)hipErrorInvalidValue;
+    case 0: ok = gemm_strided_launch<uint16_t, uint16_t, uint16_t>(d, s); break;
+    case 1: ok = gemm_strided_launch<uint16_t, uint16_t, float>(d, s); break;
+    case 4: ok = gemm_strided_launch<float, uint16_t, uint16_t>(d, s); break;
+    case 5: ok = gemm_strided_launch<float, uint16_t, float>(d, s); break;
+    case 7: ok = gemm_strided_launch<float, float, float>(d, s); break;
+    default: break;
   }
+  if (!ok) return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();
 }

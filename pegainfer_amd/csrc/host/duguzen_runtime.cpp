@@ -760,14 +760,17 @@ struct Model {
     const int P = T * f.top;
     int32_t *t_group = tiles, *t_row0 = tiles + max_tiles, *t_rows = tiles + 2 * max_tiles, *n_tiles = tiles + 3 * max_tiles;
     DZ_K(pegainfer_route_sigmoid_grouped(h, w.router, w.corr, route_e, route_w, D, f.experts, f.groups, f.keep, f.top, T, dtype, S()));
-    DZ_K(pegainfer_route_sort(route_e, P, f.top, f.experts, pos_pair, pos_row, t_group, t_row0, t_rows, n_tiles, max_tiles, S()));
+    // 128-row tiles for the matrix-core form (bf16, prompt-sized steps), 64-row tiles otherwise
+    const int per_tile = dtype == PEGAINFER_DTYPE_BF16 && !plain_kernels && T > 8 && D % 8 == 0 && f.ff % 8 == 0 ? 128 : 64;
+    DZ_K(pegainfer_route_sort(route_e, P, f.top, f.experts, pos_pair, pos_row, t_group, t_row0, t_rows, n_tiles, max_tiles, per_tile, S()));
     pegainfer_gemm_desc d{};
     d.x = h; d.w = w.gate_up_e; d.y = gu;
     d.x_dtype = d.w_dtype = d.y_dtype = dtype;
     d.m = 2 * f.ff; d.k = D;
     d.x_row_stride = D; d.w_m_stride = D; d.w_k_stride = 1; d.w_group_stride = (int64_t)2 * f.ff * D;
     d.y_row_stride = 2 * f.ff;
-    d.tile_group = t_group; d.tile_row0 = t_row0; d.tile_rows = t_rows; d.n_tiles = n_tiles; d.max_tiles = (P + 63) / 64 + f.experts;
+    d.tile_group = t_group; d.tile_row0 = t_row0; d.tile_rows = t_rows; d.n_tiles = n_tiles; d.max_tiles = (P + per_tile - 1) / per_tile + f.experts;
+    d.tile_rows_cap = per_tile;
     d.x_row_index = pos_row;
     d.max_tile_rows = std::min(T, 64);   // a row chooses distinct experts: an expert never gets more pairs than there are rows
     d.plain = plain_kernels;
@@ -782,6 +785,7 @@ struct Model {
     e.tile_group = t_group; e.tile_row0 = t_row0; e.tile_rows = t_rows; e.n_tiles = n_tiles; e.max_tiles = d.max_tiles;
     e.y_row_index = pos_pair;
     e.max_tile_rows = d.max_tile_rows;
+    e.tile_rows_cap = per_tile;
     e.plain = plain_kernels;
     DZ_K(pegainfer_gemm_strided(&e, S()));
     DZ_K(pegainfer_route_combine(ypairs, route_w, y, D, f.top, T, dtype, S()));

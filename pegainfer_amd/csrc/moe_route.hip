@@ -7,7 +7,7 @@
 //                   ties go to the lower index.
 //   sort_kernel     (row, choice) pairs bucketed by expert with LDS counters, an exclusive scan, and the table of <= 64-row
 //                   tiles the grouped GEMM walks.  The order of pairs inside an expert comes from atomics; every pair owns
-//                   its output row, so results do not depend on it.
+//                   its output row, so results do not depend on it.  Tiles hold <= 64 or <= 128 rows, as the GEMM form that walks them wants.
 //   combine_kernel  out[row] = sum over the row's choices, in choice order, of weight * expert output (fp32 sum).
 #include "common.h"
 #include "typed.h"
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restri
                                                          int32_t* __restrict__ pos_pair, int32_t* __restrict__ pos_row,
                                                          int32_t* __restrict__ tile_group, int32_t* __restrict__ tile_row0,
                                                          int32_t* __restrict__ tile_rows, int32_t* __restrict__ n_tiles,
-                                                         int max_tiles) {
+                                                         int max_tiles, int per_tile) {
   extern __shared__ int cnt[];   // [E] counts, then [E] cursors
   int* cur = cnt + E;
   for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
@@ -114,10 +114,10 @@ __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restri
     for (int e = 0; e < E; ++e) {
       const int c = cnt[e];
       cur[e] = off;
-      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += 64, ++nt) {
+      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += per_tile, ++nt) {
         tile_group[nt] = e;
         tile_row0[nt] = off + r0;
-        tile_rows[nt] = min(64, c - r0);
+        tile_rows[nt] = min(per_tile, c - r0);
       }
       off += c;
     }
@@ -169,13 +169,14 @@ pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_
 
 pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, int32_t top, int32_t experts,
                                         int32_t* pos_pair, int32_t* pos_row, int32_t* tile_group, int32_t* tile_row0,
-                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles,
+                                        int32_t* tile_rows, int32_t* n_tiles, int32_t max_tiles, int32_t rows_per_tile,
                                         pegainfer_stream_t stream) {
   if (n_pairs <= 0) return 0;
-  if (experts <= 0 || experts > 7000 || max_tiles < (n_pairs + 63) / 64 + experts)
+  if ((rows_per_tile != 64 && rows_per_tile != 128) || experts <= 0 || experts > 7000 ||
+      max_tiles < (n_pairs + rows_per_tile - 1) / rows_per_tile + experts)
     return (pegainfer_status_t)hipErrorInvalidValue;
   route_sort_kernel<<<1, 256, (size_t)2 * experts * sizeof(int), as_stream(stream)>>>(
-      expert, n_pairs, top, experts, pos_pair, pos_row, tile_group, tile_row0, tile_rows, n_tiles, max_tiles);
+      expert, n_pairs, top, experts, pos_pair, pos_row, tile_group, tile_row0, tile_rows, n_tiles, max_tiles, rows_per_tile);
   return (pegainfer_status_t)hipGetLastError();
 }
 

@@ -33,7 +33,8 @@ class GemmDesc(ctypes.Structure):
                 ("n_tiles", ctypes.c_void_p), ("max_tiles", ctypes.c_int32),
                 ("x_row_index", ctypes.c_void_p), ("y_row_index", ctypes.c_void_p),
                 ("epilogue", ctypes.c_int32), ("gate", ctypes.c_void_p), ("gate_dtype", ctypes.c_int32),
-                ("gate_row_stride", ctypes.c_int64), ("max_tile_rows", ctypes.c_int32), ("plain", ctypes.c_int32)]
+                ("gate_row_stride", ctypes.c_int64), ("max_tile_rows", ctypes.c_int32), ("tile_rows_cap", ctypes.c_int32),
+                ("plain", ctypes.c_int32)]
 
 
 def embed_f32(embed, token_ids_u32):
@@ -135,17 +136,17 @@ def route(h, w_router, correction, n_groups, keep_groups, top):
     return e, w
 
 
-def route_sort(expert, experts):
+def route_sort(expert, experts, rows_per_tile=64):
     """-> pos_pair, pos_row, tile_group, tile_row0, tile_rows, n_tiles (int32 device tensors), max_tiles"""
     rows, top = expert.shape
     P = rows * top
-    max_tiles = (P + 63) // 64 + experts
+    max_tiles = (P + rows_per_tile - 1) // rows_per_tile + experts
     dev = expert.device
     pos_pair, pos_row = torch.empty(P, dtype=torch.int32, device=dev), torch.empty(P, dtype=torch.int32, device=dev)
     tg, t0, tr = (torch.zeros(max_tiles, dtype=torch.int32, device=dev) for _ in range(3))
     nt = torch.zeros(1, dtype=torch.int32, device=dev)
     _chk(ffi.lib().pegainfer_route_sort(_p(expert), P, top, experts, _p(pos_pair), _p(pos_row), _p(tg), _p(t0), _p(tr), _p(nt),
-                                        max_tiles, _stream()), "route_sort")
+                                        max_tiles, rows_per_tile, _stream()), "route_sort")
     return pos_pair, pos_row, tg, t0, tr, nt, max_tiles
 
 

@@ -347,3 +347,28 @@ def test_strided_gemm_forms_agree(dtype):
         outs.append(y.cpu())
     ref = torch.einsum("pd,pfd->pf", x.double().repeat_interleave(top, 0), w.double()[expert.reshape(-1).long()])
     assert (outs[0].double() - ref).abs().max() < 1e-4 and (outs[1].double() - ref).abs().max() < 1e-4
+
+
+def test_grouped_gemm_over_128_row_tiles():
+    from pegainfer_amd import ops_blocks as B
+    g = torch.Generator().manual_seed(11)
+    rows, top, E, d, ff = 400, 2, 3, 64, 136         # ~267 pairs per expert: two full 128-row tiles and a part of a third
+    expert = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(rows)]).int()
+    pos_pair, pos_row, tg, t0, tr, nt, max_tiles = B.route_sort(expert.cuda(), E, rows_per_tile=128)
+    assert int(tr.cpu()[:int(nt.item())].max()) == 128
+    x, w = C.bf16_round(torch.randn(rows, d, generator=g)), C.bf16_round(torch.randn(E, ff, d, generator=g))
+    xd, wd = dev(x, torch.bfloat16), dev(w, torch.bfloat16)
+    y = torch.zeros(rows * top, ff, device="cuda")
+    B.gemm_strided(B.GemmDesc(x=xd.data_ptr(), w=wd.data_ptr(), y=y.data_ptr(), x_dtype=0, w_dtype=0, y_dtype=1, m=ff, k=d,
+                              x_row_stride=d, w_m_stride=d, w_k_stride=1, w_group_stride=ff * d, y_row_stride=ff,
+                              tile_group=tg.data_ptr(), tile_row0=t0.data_ptr(), tile_rows=tr.data_ptr(), n_tiles=nt.data_ptr(),
+                              max_tiles=max_tiles, x_row_index=pos_row.data_ptr(), y_row_index=pos_pair.data_ptr(),
+                              tile_rows_cap=128))
+    ref = torch.einsum("pd,pfd->pf", x.double().repeat_interleave(top, 0), w.double()[expert.reshape(-1).long()])
+    assert (y.cpu().double() - ref).abs().max() < 1e-4
+    with pytest.raises(RuntimeError):                 # the 64-row fp32-FMA form refuses a table cut for 128-row tiles
+        B.gemm_strided(B.GemmDesc(x=xd.data_ptr(), w=wd.data_ptr(), y=y.data_ptr(), x_dtype=0, w_dtype=0, y_dtype=1, m=ff, k=d,
+                                  x_row_stride=d, w_m_stride=d, w_k_stride=1, w_group_stride=ff * d, y_row_stride=ff,
+                                  tile_group=tg.data_ptr(), tile_row0=t0.data_ptr(), tile_rows=tr.data_ptr(),
+                                  n_tiles=nt.data_ptr(), max_tiles=max_tiles, x_row_index=pos_row.data_ptr(),
+                                  y_row_index=pos_pair.data_ptr(), tile_rows_cap=128, plain=1))
