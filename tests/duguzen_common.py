@@ -45,6 +45,13 @@ def config_b():
             "layers": [layer(m0, moe(16, 5, 1)), layer(m1, moe(40, 4, 3, count=4, keep=4)), layer(m1, dense(20))]}
 
 
+def config_odd():
+    """nothing is a multiple of 8: every vector path and matrix-core form has to step aside for its scalar / plain twin"""
+    m0, m1 = mixer(3, 10, 6, 14, 7, base=50.0, dims=4), mixer(5, 6, 2, 9, 11)
+    return {"architecture": "Duguzen", "width": 50, "vocab": 61, "norm": {"eps": 1e-5},
+            "layers": [layer(m0, dense(30)), layer(m1, moe(10, 6, 2, count=2, keep=1)), layer(m0, dense(30), 0)]}
+
+
 def config_tiny():
     return {"architecture": "Duguzen", "width": 48, "vocab": 50, "norm": {"eps": 1e-5},
             "layers": [layer(mixer(2, 8, 8, 16, 8), dense(32)), layer(mixer(2, 8, 8, 16, 8), moe(16, 4, 2, count=2, keep=1))]}

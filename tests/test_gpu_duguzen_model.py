@@ -13,7 +13,7 @@ import duguzen_common as C
 
 pytestmark = pytest.mark.gpu
 
-CONFIGS = {"a": C.config_a, "b": C.config_b, "tiny": C.config_tiny}
+CONFIGS = {"a": C.config_a, "b": C.config_b, "tiny": C.config_tiny, "odd": C.config_odd}
 
 
 def check(got, ref, dtype, what=""):
@@ -28,7 +28,7 @@ def check(got, ref, dtype, what=""):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "odd", "tiny"])
 def test_whole_prompt_every_position_and_every_layer(name, dtype):
     cfg = CONFIGS[name]()
     w = C.random_weights(cfg, 11)
@@ -57,8 +57,9 @@ def test_whole_prompt_every_position_and_every_layer(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_prefill_then_token_by_token(dtype):
-    cfg = C.config_a()
+@pytest.mark.parametrize("name", ["a", "odd"])
+def test_prefill_then_token_by_token(name, dtype):
+    cfg = CONFIGS[name]()
     w = C.random_weights(cfg, 12)
     toks = C.tokens_for(cfg, 60, 2)
     ref = C.oracle_logits(cfg, w, toks)
