@@ -573,7 +573,7 @@ struct Model {
     if (ensure_rows(T) || ensure_want((size_t)std::max(1, W))) return -1;
     // decode-like steps (few rows) cut the keys finely so that one request's context spreads over many workgroups;
     // prompt-sized steps have rows enough and only cut very long contexts
-    const int split_keys = T * (size_t)mx_heads <= 1024 ? 64 : 4096;
+    const int split_keys = T * (size_t)mx_heads <= 1024 ? 32 : 4096;
     const int64_t ws_need = pegainfer_latent_attention_workspace((int)T, mx_heads, mx_rank, max_kv, split_keys);
     if ((size_t)ws_need > attn_ws_cap) {
       DZ_HIP(hipStreamSynchronize(stream));

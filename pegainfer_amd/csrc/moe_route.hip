@@ -3,8 +3,8 @@
 //   route_kernel    one workgroup per token row: fp32 router logits (a wave per expert, lanes over the width), sigmoid
 //                   scores, the correction added for the CHOICE only, group scores = the two largest choices of a group,
 //                   the best `keep` groups stay eligible, then the `top` largest eligible choices; weights = the plain
-//                   sigmoid scores of the chosen experts.  Selection is serial in one thread: E is tens to hundreds, and
-//                   ties go to the lower index.
+//                   sigmoid scores of the chosen experts.  Selection runs on one wave: a lane per group for the group
+//                   scores and ranks, then `top` wave-wide arg-max steps; ties go to the lower index.
 //   sort_kernel     (row, choice) pairs bucketed by expert with LDS counters, an exclusive scan, and the table of <= 64-row
 //                   tiles the grouped GEMM walks.  The order of pairs inside an expert comes from atomics; every pair owns
 //                   its output row, so results do not depend on it.  Tiles hold <= 64 or <= 128 rows, as the GEMM form that walks them wants.
@@ -61,10 +61,11 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
     }
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
+  if (wave != 0) return;
+  // ---- selection by wave 0 alone: LDS accesses of one wave complete in order, so no barrier is needed between its steps
   if (G > 1) {
     const int per = E / G;
-    for (int g = 0; g < G; ++g) {
+    for (int g = lane; g < G; g += 64) {             // a lane scores a group: its two largest choices
       float b0 = -INFINITY, b1 = -INFINITY;
       for (int i = 0; i < per; ++i) {
         const float v = ch[g * per + i];
@@ -72,29 +73,39 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
       }
       gs[g] = per >= 2 ? b0 + b1 : b0;
     }
-    // drop the G - keep worst groups: repeatedly take the best remaining group, mark it kept (score := NaN-free flag)
-    for (int k = 0; k < keep; ++k) {
-      int best = -1;
-      for (int g = 0; g < G; ++g)
-        if (gs[g] != INFINITY && (best < 0 || gs[g] > gs[best])) best = g;
-      if (best >= 0) gs[best] = INFINITY;   // kept
-    }
-    for (int g = 0; g < G; ++g)
-      if (gs[g] != INFINITY)
+    __builtin_amdgcn_wave_barrier();
+    for (int g = lane; g < G; g += 64) {             // kept = fewer than `keep` groups rank ahead (ties: the lower index)
+      const float mine = gs[g];
+      int ahead = 0;
+      for (int o = 0; o < G; ++o) {
+        const float v = gs[o];
+        ahead += (v > mine || (v == mine && o < g)) ? 1 : 0;
+      }
+      if (ahead >= keep)
         for (int i = 0; i < per; ++i) ch[g * per + i] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
   }
   for (int k = 0; k < top; ++k) {
-    int best = 0;
     float bv = -INFINITY;
-    bool found = false;
-    for (int e = 0; e < E; ++e) {
+    int be = 0x7FFFFFFF;
+    for (int e = lane; e < E; e += 64) {             // ascending e per lane: the first maximum is the lowest index
       const float v = ch[e];
-      if (v == -INFINITY) continue;         // taken or not eligible
-      if (!found || v > bv) { best = e; bv = v; found = true; }
+      if (v > bv) { bv = v; be = e; }
     }
-    out_e[(size_t)row * top + k] = best;
-    out_w[(size_t)row * top + k] = found ? s[best] : 0.f;
-    if (found) ch[best] = -INFINITY;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, kWave);
+      const int oe = __shfl_xor(be, off, kWave);
+      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+    }
+    const bool found = bv != -INFINITY;
+    if (lane == 0) {
+      out_e[(size_t)row * top + k] = found ? be : 0;
+      out_w[(size_t)row * top + k] = found ? s[be] : 0.f;
+      if (found) ch[be] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
