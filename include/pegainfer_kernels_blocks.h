@@ -140,6 +140,108 @@ pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, 
 pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,
                                            int32_t rows, int32_t dtype, pegainfer_stream_t stream);
 
+/* ---- sequences with state: ragged batches ----
+ * A step's token rows are the concatenation of its entries; entry e owns rows entry_row0[e] .. entry_row0[e + 1] - 1 and
+ * the state slot entry_slot[e].  Per-slot state lives in fp32 at  state + slot * slot_stride  (floats). */
+
+/* Causal per-channel convolution over time with carried inputs:
+ *   out[t, c] = (mode & 1 ? in[t, c] : 0) + sum_j w[c, j] * in[t - taps + 1 + j, c]      (mode & 2: silu of the whole)
+ * inputs before the entry's first row come from the slot's state (its last taps - 1 inputs, oldest first, [taps - 1][C]);
+ * before the sequence's start that state is zero.  in: fp32 or bf16 by in_dtype; w [C][taps] by w_dtype; out by out_dtype.
+ * pegainfer_time_conv only reads the state; pegainfer_time_conv_commit, enqueued after it, moves the state on by the
+ * entry's rows. */
+pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
+                                       const float* state, int64_t slot_stride, void* out, int32_t out_dtype,
+                                       int64_t out_row_stride, int32_t channels, int32_t taps, int32_t mode,
+                                       const int32_t* row_entry, const int32_t* entry_row0, const int32_t* entry_slot,
+                                       int32_t n_rows, pegainfer_stream_t stream);
+pegainfer_status_t pegainfer_time_conv_commit(const void* in, int32_t in_dtype, int64_t in_row_stride, float* state,
+                                              int64_t slot_stride, int32_t channels, int32_t taps, const int32_t* entry_row0,
+                                              const int32_t* entry_slot, int32_t n_entries, pegainfer_stream_t stream);
+
+/* RMS norm in groups on a sublayer's OUTPUT, the residual sum, and optionally a weighted sum over earlier streams:
+ *   n      = y cut into `groups` equal consecutive parts, each / sqrt(mean(part^2) + eps), whole row * w
+ *   r      = (x_in ? x_in : 0) + n                           -> x_out (fp32, optional), xb_out (dtype, optional)
+ *   mix    = sum_{j < n_mix - 1} coef[j] * stack[j * stack_stride + row * d + :] + coef[n_mix - 1] * r     -> mix_out (fp32)
+ * y by y_dtype, w and coef by dtype; everything is computed in fp32.  x_out may alias x_in; mix_out may alias x_in. */
+pegainfer_status_t pegainfer_group_rms_add(const float* x_in, const void* y, int32_t y_dtype, const void* w, int32_t groups,
+                                           float eps, float* x_out, void* xb_out, int32_t d, int32_t rows, int32_t dtype,
+                                           const float* stack, int64_t stack_stride, const void* coef, int32_t n_mix,
+                                           float* mix_out, void* mixb_out, pegainfer_stream_t stream);
+
+/* out[row, i] = g * sigmoid(alpha * g) * (u + 1),  g = min(gu[row, i], limit),  u = clamp(gu[row, I + i], -limit, limit) */
+pegainfer_status_t pegainfer_clamp_glu_rows(const void* gate_up, void* out, int32_t I, int32_t rows, float limit, float alpha,
+                                            int32_t dtype, pegainfer_stream_t stream);
+
+/* Router with a choice of score: score_kind 0 = sigmoid per expert (pegainfer_route_sigmoid_grouped), 1 = softmax over all
+ * experts.  Groups, correction, selection and weights as there. */
+enum { PEGAINFER_SCORE_SIGMOID = 0, PEGAINFER_SCORE_SOFTMAX = 1 };
+pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, const void* correction, int32_t* out_expert,
+                                        float* out_weight, int32_t d, int32_t experts, int32_t n_groups, int32_t keep_groups,
+                                        int32_t top, int32_t rows, int32_t score_kind, int32_t dtype, pegainfer_stream_t stream);
+/* pegainfer_route_combine plus a row every token gets (a shared expert's output, [rows, d] of dtype; NULL = none) */
+pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
+                                               int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream);
+
+/* ---- recurrent matrix memories (state per (slot, head): S [dim][vdim] fp32, row-major) ----
+ * Gated delta rule.  Per row, from qkv (fp32 [rows][qkv_stride]: q heads at 0, k heads at kv_heads * dim, v heads at
+ * 2 * kv_heads * dim) and the projection row `proj` (dtype; beta logits at b_off, decay inputs at a_off, one per head):
+ *   q, k -> x / sqrt(sum(x^2) + 1e-6) per head (q also * dim^-1/2);  beta = sigmoid(b);  g = exp(-exp(A_log) * softplus(a + dt_bias))
+ *   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          head h reads q / k head h / (heads / kv_heads)
+ * o: fp32 [rows][heads * vdim].  dim <= 256. */
+pegainfer_status_t pegainfer_delta_rule(const float* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
+                                        int64_t b_off, int64_t a_off, const void* A_log, const void* dt_bias, float* state,
+                                        int64_t slot_stride, float* o, int32_t heads, int32_t kv_heads, int32_t dim,
+                                        int32_t vdim, const int32_t* entry_row0, const int32_t* entry_slot, int32_t n_entries,
+                                        int32_t dtype, pegainfer_stream_t stream);
+/* Exponentially gated matrix memory with a running maximum (state per (slot, head): S [dim][vdim], n [dim], m; the slot's
+ * region is [S of all heads | n of all heads | m of all heads]).  Per row from `proj` (dtype): q at q_off, k at k_off
+ * (heads x dim), v at v_off (heads x vdim), gate inputs at i_off / f_off (one per head), biases i_bias / f_bias:
+ *   i = cap tanh((zi + bi) / cap);  f = logsigmoid(cap tanh((zf + bf) / cap));  m' = max(f + m, i)
+ *   S <- exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k;  o = S^T (q dim^-1/2) / (max(|n . q dim^-1/2|, exp(-m')) + 1e-6)
+ * m starts at 0.  o: fp32 [rows][heads * vdim].  dim <= 256. */
+pegainfer_status_t pegainfer_gated_matrix_memory(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off,
+                                                 int64_t v_off, int64_t i_off, int64_t f_off, const void* i_bias,
+                                                 const void* f_bias, float cap, float* state, int64_t slot_stride, float* o,
+                                                 int32_t heads, int32_t dim, int32_t vdim, const int32_t* entry_row0,
+                                                 const int32_t* entry_slot, int32_t n_entries, int32_t dtype,
+                                                 pegainfer_stream_t stream);
+/* Per-head RMS norm of a memory's read-out, a weight, a gate and a constant factor:
+ *   out[row, h, :] = o[row, h, :] / sqrt(mean(o[row, h, :]^2) + eps) * w * act(gate[row, h, :]) * factor
+ * w: [vdim] shared by the heads (w_per_head == 0) or [heads * vdim]; gate_kind 0 = silu, 1 = sigmoid; gate rows of dtype
+ * with stride gate_stride; out rows of dtype with stride out_stride. */
+pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_t w_per_head, const void* gate,
+                                           int64_t gate_stride, int32_t gate_kind, float factor, float eps, void* out,
+                                           int64_t out_stride, int32_t heads, int32_t vdim, int32_t rows, int32_t dtype,
+                                           pegainfer_stream_t stream);
+
+/* ---- softmax attention over a paged key/value cache, any head sizes, grouped key/value heads ----
+ * Cache: page-first; one layer's part of a page = [slot][kv_heads][dim] keys at k_off, [slot][kv_heads][vdim] values at
+ * v_off (elements of dtype from the page's start).
+ * pegainfer_qk_norm_rope_paged: per row from `proj` (dtype): q heads at q_off, k heads at k_off, v heads at v_off.
+ *   q, k -> RMS norm over dim (eps) * q_norm / k_norm ([dim], plain weight), then neighbours (2i, 2i + 1) of the first
+ *   rot_dims values rotated by position * inv_freq[i] (fp32 angles); k and v go to the cache entry of (request, position),
+ *   q to q_out (fp32 [rows][heads][dim]). */
+pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off,
+                                                int64_t v_off, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
+                                                const void* q_norm, const void* k_norm, float eps, const float* inv_freq,
+                                                int32_t rot_dims, const int32_t* positions, const int32_t* row_entry,
+                                                const int32_t* page_indptr, const int32_t* page_ids, void* cache,
+                                                int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
+                                                int32_t page_size, float* q_out, int32_t n_rows, int32_t dtype,
+                                                pegainfer_stream_t stream);
+/* Causal softmax attention, scores and weights in fp32:  out[row, h, :] = factor * sum_{j <= position} softmax_j(q . k_j * scale) v_j.
+ * The rows are cut by the caller into tiles that stay inside one entry: tile i covers rows tile_row0[i] .. + tile_ntok[i] - 1
+ * and, of each key/value group's query heads, tile_qh0[i] .. + tile_nqh[i] - 1, with ntok * nqh <= 16.  dim, vdim <= 256.
+ * out rows of dtype with stride out_stride. */
+pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, int64_t page_stride, int64_t k_cache_off,
+                                             int64_t v_cache_off, int32_t page_size, const int32_t* positions,
+                                             const int32_t* row_entry, const int32_t* page_indptr, const int32_t* page_ids,
+                                             int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float scale,
+                                             float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
+                                             const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
+                                             int64_t out_stride, int32_t dtype, pegainfer_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,6 +12,7 @@
 #include "pegainfer_qwen3.h"
 #include "pegainfer_qwen35.h"
 #include "pegainfer_duguzen.h"
+#include "pegainfer_feruzen.h"
 #include "pegainfer_scheduler.h"
 
 namespace psched {
@@ -275,25 +276,49 @@ struct Qwen35Exec {
   }
 };
 
-// Executor over the Duguzen runtime (pegainfer_duguzen.h).  Its step function takes prompts and single tokens of several
-// requests as ONE batch, so a Prefill, a Decode and a Unified plan are all the same call; sampled requests draw from their
-// wanted row afterwards, logprobs read the row's fp32 logits.
-struct DuguzenExec {
-  pegainfer_duguzen_t model;
+// Executor over a runtime with ONE batched step function (pegainfer_duguzen.h, pegainfer_feruzen.h).  The step takes prompts
+// and single tokens of several requests as ONE batch, so a Prefill, a Decode and a Unified plan are all the same call;
+// sampled requests draw from their wanted row afterwards, logprobs read the row's fp32 logits.  Api names the runtime's
+// entry points.
+#define PEGAINFER_STEP_API(NAME, PREFIX)                                                                                      \
+  struct NAME {                                                                                                                \
+    static int32_t page_size(void* m) { return PREFIX##_page_size(m); }                                                        \
+    static int32_t capacity_pages(void* m) { return PREFIX##_capacity_pages(m); }                                              \
+    static int32_t available_pages(void* m) { return PREFIX##_available_pages(m); }                                            \
+    static int32_t max_batch_size(void* m) { return PREFIX##_max_batch_size(m); }                                              \
+    static int32_t new_request(void* m) { return PREFIX##_new_request(m); }                                                    \
+    static int32_t drop_request(void* m, int32_t id) { return PREFIX##_drop_request(m, id); }                                  \
+    static const char* last_error(void* m) { return PREFIX##_last_error(m); }                                                  \
+    static int32_t step(void* m, int32_t n, const int32_t* ids, const int32_t* lens, const uint32_t* tokens, int32_t* out) {   \
+      return PREFIX##_step(m, n, ids, lens, tokens, -1, nullptr, nullptr, out);                                                \
+    }                                                                                                                          \
+    static int32_t sample(void* m, int32_t row, float t, int32_t k, float p, float rv, int32_t* out) {                         \
+      return PREFIX##_sample(m, row, t, k, p, rv, out);                                                                        \
+    }                                                                                                                          \
+    static int32_t logprobs(void* m, int32_t row, uint32_t token, int32_t k, float* lp, uint32_t* ids, float* vals) {          \
+      return PREFIX##_logprobs(m, row, token, k, lp, ids, vals);                                                               \
+    }                                                                                                                          \
+  }
+PEGAINFER_STEP_API(DuguzenApi, pegainfer_duguzen);
+PEGAINFER_STEP_API(FeruzenApi, pegainfer_feruzen);
+
+template <class Api>
+struct StepExec {
+  void* model;
   std::unordered_set<uint32_t> stop;
   std::unordered_map<uint64_t, int32_t> slot;
   std::string err;
-  static DuguzenExec* E(void* u) { return (DuguzenExec*)u; }
-  static int32_t page_size(void* u) { return pegainfer_duguzen_page_size(E(u)->model); }
-  static int32_t max_request_pages(void* u) { return pegainfer_duguzen_capacity_pages(E(u)->model); }
-  static int32_t available_pages(void* u) { return pegainfer_duguzen_available_pages(E(u)->model); }
-  static int32_t max_batch_size(void* u) { return pegainfer_duguzen_max_batch_size(E(u)->model); }
+  static StepExec* E(void* u) { return (StepExec*)u; }
+  static int32_t page_size(void* u) { return Api::page_size(E(u)->model); }
+  static int32_t max_request_pages(void* u) { return Api::capacity_pages(E(u)->model); }
+  static int32_t available_pages(void* u) { return Api::available_pages(E(u)->model); }
+  static int32_t max_batch_size(void* u) { return Api::max_batch_size(E(u)->model); }
   static int32_t is_stop_token(void* u, uint32_t t) { return E(u)->stop.count(t) ? 1 : 0; }
   static int32_t drop_request(void* u, uint64_t id) {
     auto* e = E(u);
     auto it = e->slot.find(id);
     if (it == e->slot.end()) return 0;
-    const int32_t rc = pegainfer_duguzen_drop_request(e->model, it->second);
+    const int32_t rc = Api::drop_request(e->model, it->second);
     e->slot.erase(it);
     return rc;
   }
@@ -304,7 +329,7 @@ struct DuguzenExec {
                          const float* rv, uint32_t* out) {
     auto* e = E(u);
     auto fail = [&](const char* what) {
-      const char* m = pegainfer_duguzen_last_error(e->model);
+      const char* m = Api::last_error(e->model);
       e->err = std::string(what) + ": " + (m ? m : "");
       return -1;
     };
@@ -312,7 +337,7 @@ struct DuguzenExec {
     std::vector<int32_t> slots(n), toks(n);
     for (int i = 0; i < n; ++i) {
       if (i < n_pf) {
-        const int32_t r = pegainfer_duguzen_new_request(e->model);
+        const int32_t r = Api::new_request(e->model);
         if (r < 0) return fail("new_request");
         e->slot[ids[i]] = r;
         slots[i] = r;
@@ -322,10 +347,10 @@ struct DuguzenExec {
         slots[i] = it->second;
       }
     }
-    if (pegainfer_duguzen_step(e->model, n, slots.data(), lens, tokens, -1, nullptr, nullptr, toks.data())) return fail("step");
+    if (Api::step(e->model, n, slots.data(), lens, tokens, toks.data())) return fail("step");
     for (int i = 0; i < n; ++i) {
       if (!greedy(temp[i], top_k[i], top_p[i]) &&
-          pegainfer_duguzen_sample(e->model, i, temp[i], top_k[i], top_p[i], rv[i], &toks[i]))
+          Api::sample(e->model, i, temp[i], top_k[i], top_p[i], rv[i], &toks[i]))
         return fail("sample");
       out[i] = (uint32_t)toks[i];
     }
@@ -333,17 +358,20 @@ struct DuguzenExec {
   }
   static int32_t logprobs(void* u, int32_t row, uint32_t token, int32_t top_k, float* lp, uint32_t* ids, float* vals) {
     auto* e = E(u);
-    const int32_t rc = pegainfer_duguzen_logprobs(e->model, row, token, top_k, lp, ids, vals);
-    if (rc < 0) { const char* m = pegainfer_duguzen_last_error(e->model); e->err = m ? m : "logprobs failed"; }
+    const int32_t rc = Api::logprobs(e->model, row, token, top_k, lp, ids, vals);
+    if (rc < 0) { const char* m = Api::last_error(e->model); e->err = m ? m : "logprobs failed"; }
     return rc;
   }
 };
+using DuguzenExec = StepExec<DuguzenApi>;
+using FeruzenExec = StepExec<FeruzenApi>;
 
 struct Scheduler {
   pegainfer_executor_vtbl ex;
   Qwen3Exec* owned = nullptr;
   Qwen35Exec* owned35 = nullptr;
   DuguzenExec* owned_dz = nullptr;
+  FeruzenExec* owned_fz = nullptr;
   Rng rng;
   std::vector<Active> active;
   std::vector<Pending> deferred;
@@ -613,11 +641,25 @@ pegainfer_sched_t pegainfer_sched_create_duguzen(void* model, uint64_t seed, con
   s->owned_dz = e;
   return s;
 }
+pegainfer_sched_t pegainfer_sched_create_feruzen(void* model, uint64_t seed, const uint32_t* stop_tokens, int32_t n_stop) {
+  if (!model) return nullptr;
+  auto* e = new psched::FeruzenExec();
+  e->model = model;
+  for (int i = 0; i < n_stop; ++i) e->stop.insert(stop_tokens[i]);
+  pegainfer_executor_vtbl v{sizeof(pegainfer_executor_vtbl), e, &psched::FeruzenExec::page_size, &psched::FeruzenExec::max_request_pages,
+                            &psched::FeruzenExec::available_pages, &psched::FeruzenExec::is_stop_token,
+                            &psched::FeruzenExec::drop_request, &psched::FeruzenExec::execute, &psched::FeruzenExec::last_error,
+                            &psched::FeruzenExec::max_batch_size, &psched::FeruzenExec::logprobs, nullptr, nullptr};
+  Scheduler* s = static_cast<Scheduler*>(pegainfer_sched_create(&v, seed));
+  s->owned_fz = e;
+  return s;
+}
 void pegainfer_sched_destroy(pegainfer_sched_t s) {
   if (!s) return;
   delete SC(s)->owned;
   delete SC(s)->owned35;
   delete SC(s)->owned_dz;
+  delete SC(s)->owned_fz;
   delete SC(s);
 }
 uint64_t pegainfer_sched_submit_ex(pegainfer_sched_t s, const uint32_t* prompt_tokens, int32_t n_tokens, int32_t max_tokens,

@@ -18,7 +18,8 @@ namespace pk {
 template <typename A>
 __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, const A* __restrict__ wr,
                                                     const A* __restrict__ corr, int32_t* __restrict__ out_e,
-                                                    float* __restrict__ out_w, int d, int E, int G, int keep, int top) {
+                                                    float* __restrict__ out_w, int d, int E, int G, int keep, int top,
+                                                    int score) {
   extern __shared__ float sm[];
   float* s = sm;            // [E] sigmoid scores
   float* ch = sm + E;       // [E] choice scores (eligible) or -inf
@@ -54,7 +55,7 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
       const float z = wave_sum(a[q]);
       const int e = e0 + q;
       if (lane == 0 && e < E) {
-        const float sc = sigmoid_f(z);
+        const float sc = score == PEGAINFER_SCORE_SOFTMAX ? z : sigmoid_f(z);   // softmax: the logit for now
         s[e] = sc;
         ch[e] = corr ? sc + ld(corr + e) : sc;
       }
@@ -63,6 +64,20 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
   __syncthreads();
   if (wave != 0) return;
   // ---- selection by wave 0 alone: LDS accesses of one wave complete in order, so no barrier is needed between its steps
+  if (score == PEGAINFER_SCORE_SOFTMAX) {            // s = exp(z - max) / sum over ALL experts, then the choice scores
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) sum += expf(s[e] - mx);
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+      const float sc = expf(s[e] - mx) / sum;
+      s[e] = sc;
+      ch[e] = corr ? sc + ld(corr + e) : sc;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
   if (G > 1) {
     const int per = E / G;
     for (int g = lane; g < G; g += 64) {             // a lane scores a group: its two largest choices
@@ -144,10 +159,10 @@ __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restri
 
 template <typename A>
 __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
-                                                            A* __restrict__ out, int d, int top) {
+                                                            const A* __restrict__ add, A* __restrict__ out, int d, int top) {
   const int row = blockIdx.x;
   for (int i = threadIdx.x; i < d; i += 256) {
-    float a = 0.f;
+    float a = add ? ld(add + (size_t)row * d + i) : 0.f;
     for (int c = 0; c < top; ++c) a = fmaf(w[(size_t)row * top + c], y[((size_t)row * top + c) * d + i], a);
     st(out + (size_t)row * d + i, a);
   }
@@ -158,11 +173,11 @@ __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restr
 extern "C" {
 using namespace pk;
 
-pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_router, const void* correction,
-                                                   int32_t* out_expert, float* out_weight, int32_t d, int32_t experts,
-                                                   int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
-                                                   int32_t dtype, pegainfer_stream_t stream) {
+pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, const void* correction, int32_t* out_expert,
+                                        float* out_weight, int32_t d, int32_t experts, int32_t n_groups, int32_t keep_groups,
+                                        int32_t top, int32_t rows, int32_t score_kind, int32_t dtype, pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
+  if (score_kind != PEGAINFER_SCORE_SIGMOID && score_kind != PEGAINFER_SCORE_SOFTMAX) return (pegainfer_status_t)hipErrorInvalidValue;
   if (n_groups < 1) n_groups = 1;
   if (experts <= 0 || experts % n_groups || top <= 0 || top > experts || keep_groups < 1 || keep_groups > n_groups ||
       (size_t)(2 * experts + n_groups) * 4 > 60000)
@@ -172,10 +187,18 @@ pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_
         using A = std::remove_pointer_t<decltype(t)>;
         route_kernel<A><<<rows, 256, smem, as_stream(stream)>>>(static_cast<const A*>(h), static_cast<const A*>(w_router),
                                                                 static_cast<const A*>(correction), out_expert, out_weight, d,
-                                                                experts, n_groups, keep_groups, top);
+                                                                experts, n_groups, keep_groups, top, score_kind);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_sigmoid_grouped(const void* h, const void* w_router, const void* correction,
+                                                   int32_t* out_expert, float* out_weight, int32_t d, int32_t experts,
+                                                   int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                                   int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_route_topk(h, w_router, correction, out_expert, out_weight, d, experts, n_groups, keep_groups, top, rows,
+                              PEGAINFER_SCORE_SIGMOID, dtype, stream);
 }
 
 pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, int32_t top, int32_t experts,
@@ -191,15 +214,21 @@ pegainfer_status_t pegainfer_route_sort(const int32_t* expert, int32_t n_pairs, 
   return (pegainfer_status_t)hipGetLastError();
 }
 
-pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,
-                                           int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
+pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
+                                               int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
   if (!by_dtype(dtype, [&](auto* t) {
         using A = std::remove_pointer_t<decltype(t)>;
-        route_combine_kernel<A><<<rows, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<A*>(out), d, top);
+        route_combine_kernel<A><<<rows, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<const A*>(add),
+                                                                     static_cast<A*>(out), d, top);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_combine(const float* y_pairs, const float* weight, void* out, int32_t d, int32_t top,
+                                           int32_t rows, int32_t dtype, pegainfer_stream_t stream) {
+  return pegainfer_route_combine_add(y_pairs, weight, nullptr, out, d, top, rows, dtype, stream);
 }
 
 }  // extern "C"

@@ -58,7 +58,8 @@ class Scheduler:
         lib = ffi.host_lib()
         st = np.ascontiguousarray(list(stop_tokens), dtype=np.uint32)
         create = {"Qwen35Engine": lib.pegainfer_sched_create_qwen35,
-                  "DuguzenEngine": lib.pegainfer_sched_create_duguzen}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
+                  "DuguzenEngine": lib.pegainfer_sched_create_duguzen,
+                  "FeruzenEngine": lib.pegainfer_sched_create_feruzen}.get(type(engine).__name__, lib.pegainfer_sched_create_qwen3)
         h = create(engine.h, seed, st.ctypes.data if st.size else None, int(st.size))
         return cls(h, keep=engine)
 
