@@ -1,6 +1,7 @@
 """Torch-tensor wrappers over include/pegainfer_kernels_blocks.h: the model-independent blocks that exist in a bf16 and a
 true-fp32 instance (Dynamic-Tanh norms over an fp32 stream, activations, the strided / batched / grouped GEMM, attention
-over a paged latent cache, sigmoid-scored grouped routing).  Tensors are torch CUDA tensors used as device memory; the
+over a paged latent cache, routing; time convolutions with carried tails, grouped output norms with a depth-weighted
+sum, clamp-GLU, recurrent matrix memories over per-request state, attention over a paged key/value cache).  Tensors are torch CUDA tensors used as device memory; the
 storage type of a call (bf16 / fp32) is taken from the activation tensor.  Work is enqueued on torch's current stream.
 No CPU fallback: without the HIP library every call raises ImportError.
 """
@@ -155,4 +156,146 @@ def route_combine(y_pairs, weight, out_dtype):
     d = y_pairs.shape[1]
     out = torch.empty((rows, d), dtype=out_dtype, device=y_pairs.device)
     _chk(ffi.lib().pegainfer_route_combine(_p(y_pairs), _p(weight), _p(out), d, top, rows, _dt(out), _stream()), "route_combine")
+    return out
+
+
+# ---- sequences with state: ragged batches (entry e = rows entry_row0[e] .. entry_row0[e + 1] - 1, state slot entry_slot[e]) ----
+class Ragged:
+    """device index arrays of a step whose entries have `lens` rows and use the state slots `slots`; positions start at
+    `starts` (default 0)"""
+
+    def __init__(self, lens, slots=None, starts=None, device="cuda"):
+        slots = list(range(len(lens))) if slots is None else slots
+        starts = [0] * len(lens) if starts is None else starts
+        row0, ent, pos = [0], [], []
+        for i, n in enumerate(lens):
+            row0.append(row0[-1] + n)
+            ent += [i] * n
+            pos += list(range(starts[i], starts[i] + n))
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
+        self.lens, self.n, self.rows = list(lens), len(lens), row0[-1]
+        self.entry_row0, self.entry_slot, self.row_entry, self.positions = i32(row0), i32(slots), i32(ent), i32(pos)
+
+
+def time_conv(x, w, state, rg, residual=False, silu=False, out_dtype=None, channels=None):
+    """causal per-channel convolution over time; state fp32 [slots, taps - 1, C] is read, then moved on by the step's rows"""
+    C = channels or w.shape[0]
+    taps = w.shape[1]
+    out = torch.empty((x.shape[0], C), dtype=out_dtype or x.dtype, device=x.device)
+    slot_stride = state.shape[1] * state.shape[2] if state.dim() == 3 else 0
+    L = ffi.lib()
+    _chk(L.pegainfer_time_conv(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(state), slot_stride, _p(out), _dt(out), C, C, taps,
+                               (1 if residual else 0) | (2 if silu else 0), _p(rg.row_entry), _p(rg.entry_row0),
+                               _p(rg.entry_slot), x.shape[0], _stream()), "time_conv")
+    _chk(L.pegainfer_time_conv_commit(_p(x), _dt(x), x.stride(0), _p(state), slot_stride, C, taps, _p(rg.entry_row0),
+                                      _p(rg.entry_slot), rg.n, _stream()), "time_conv_commit")
+    return out
+
+
+def group_rms_add(y, w, groups, eps, x=None, stack=None, coef=None):
+    """r = (x or 0) + grouped_rms(y) * w  -> (r fp32, r in w's dtype, mix fp32 or None) with
+    mix = sum_j coef[j] stack[j] + coef[-1] r over the len(coef) - 1 streams of `stack` (fp32 [n, rows, d])"""
+    rows, d = y.shape
+    r32 = torch.empty((rows, d), dtype=torch.float32, device=y.device)
+    rb = torch.empty((rows, d), dtype=w.dtype, device=y.device)
+    n_mix = 0 if coef is None else coef.numel()
+    mix = torch.empty((rows, d), dtype=torch.float32, device=y.device) if n_mix else None
+    _chk(ffi.lib().pegainfer_group_rms_add(_p(x), _p(y), _dt(y), _p(w), groups, float(eps), _p(r32), _p(rb), d, rows, _dt(w),
+                                           _p(stack), 0 if stack is None else stack.stride(0), _p(coef), n_mix, _p(mix), None,
+                                           _stream()), "group_rms_add")
+    return r32, rb, mix
+
+
+def clamp_glu_rows(gate_up, limit, alpha=1.702):
+    rows, two_i = gate_up.shape
+    out = torch.empty((rows, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _chk(ffi.lib().pegainfer_clamp_glu_rows(_p(gate_up), _p(out), two_i // 2, rows, float(limit), float(alpha), _dt(gate_up),
+                                            _stream()), "clamp_glu_rows")
+    return out
+
+
+def route_topk(h, w_router, top, score="softmax", correction=None, n_groups=1, keep_groups=1):
+    rows, d = h.shape
+    e = torch.empty((rows, top), dtype=torch.int32, device=h.device)
+    w = torch.empty((rows, top), dtype=torch.float32, device=h.device)
+    _chk(ffi.lib().pegainfer_route_topk(_p(h), _p(w_router), _p(correction), _p(e), _p(w), d, w_router.shape[0], n_groups,
+                                        keep_groups, top, rows, 1 if score == "softmax" else 0, _dt(h), _stream()), "route_topk")
+    return e, w
+
+
+def route_combine_add(y_pairs, weight, add, out_dtype):
+    rows, top = weight.shape
+    d = y_pairs.shape[1]
+    out = torch.empty((rows, d), dtype=out_dtype, device=y_pairs.device)
+    _chk(ffi.lib().pegainfer_route_combine_add(_p(y_pairs), _p(weight), _p(add), _p(out), d, top, rows, _dt(out), _stream()),
+         "route_combine_add")
+    return out
+
+
+def delta_rule(qkv_f32, proj, b_off, a_off, A_log, dt_bias, state, heads, kv_heads, dim, vdim, rg):
+    """qkv fp32 [rows, 2 kv dim + heads vdim] (after convolution and silu), proj [rows, *] with the beta / decay inputs;
+    state fp32 [slots, heads, dim, vdim] is updated in place; returns o fp32 [rows, heads * vdim]"""
+    o = torch.empty((qkv_f32.shape[0], heads * vdim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_delta_rule(_p(qkv_f32), qkv_f32.stride(0), _p(proj), proj.stride(0), b_off, a_off, _p(A_log),
+                                        _p(dt_bias), _p(state), state.stride(0), _p(o), heads, kv_heads, dim, vdim,
+                                        _p(rg.entry_row0), _p(rg.entry_slot), rg.n, _dt(proj), _stream()), "delta_rule")
+    return o
+
+
+def gated_matrix_memory(proj, offs, i_bias, f_bias, cap, state, heads, dim, vdim, rg):
+    """proj [rows, *] with q / k / v / i / f at the column offsets `offs`; state fp32 [slots, heads (dim vdim + dim + 1)] laid
+    out [S of all heads | n of all heads | m of all heads]; returns o fp32 [rows, heads * vdim]"""
+    o = torch.empty((proj.shape[0], heads * vdim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_gated_matrix_memory(_p(proj), proj.stride(0), offs[0], offs[1], offs[2], offs[3], offs[4], _p(i_bias),
+                                                 _p(f_bias), float(cap), _p(state), state.stride(0), _p(o), heads, dim, vdim,
+                                                 _p(rg.entry_row0), _p(rg.entry_slot), rg.n, _dt(proj), _stream()),
+         "gated_matrix_memory")
+    return o
+
+
+def head_rms_gate(o_f32, w, gate, gate_kind, factor, eps, heads, vdim, out=None):
+    """gate: a [rows, heads * vdim] view (row stride free) in w's dtype; gate_kind "silu" | "sigmoid" """
+    rows = o_f32.shape[0]
+    out = torch.empty((rows, heads * vdim), dtype=w.dtype, device=w.device) if out is None else out
+    _chk(ffi.lib().pegainfer_head_rms_gate(_p(o_f32), _p(w), int(w.numel() != vdim),
+                                           _p(gate), gate.stride(0), 0 if gate_kind == "silu" else 1, float(factor), float(eps),
+                                           _p(out), out.stride(0), heads, vdim, rows, _dt(w), _stream()), "head_rms_gate")
+    return out
+
+
+def attention_tiles(lens, per_group, device="cuda"):
+    """row tiles of pegainfer_paged_attention for entries of `lens` rows: runs of token rows times runs of the per_group query
+    heads of a key/value head, at most 16 rows each"""
+    row0, ntok, qh0, nqh, at = [], [], [], [], 0
+    for n in lens:
+        if per_group <= 16:
+            tpt = 16 // per_group
+            for t0 in range(0, n, tpt):
+                row0.append(at + t0); ntok.append(min(tpt, n - t0)); qh0.append(0); nqh.append(per_group)  # noqa: E702
+        else:
+            for t0 in range(n):
+                for q0 in range(0, per_group, 16):
+                    row0.append(at + t0); ntok.append(1); qh0.append(q0); nqh.append(min(16, per_group - q0))  # noqa: E702
+        at += n
+    return tuple(torch.tensor(v, dtype=torch.int32, device=device) for v in (row0, ntok, qh0, nqh))
+
+
+def qk_norm_rope_paged(proj, offs, heads, kv_heads, dim, vdim, q_norm, k_norm, eps, inv_freq, rot_dims, rg, page_indptr,
+                       page_ids, cache, page_stride, k_off, v_off, page_size):
+    q = torch.empty((proj.shape[0], heads, dim), dtype=torch.float32, device=proj.device)
+    _chk(ffi.lib().pegainfer_qk_norm_rope_paged(_p(proj), proj.stride(0), offs[0], offs[1], offs[2], heads, kv_heads, dim, vdim,
+                                                _p(q_norm), _p(k_norm), float(eps), _p(inv_freq), rot_dims, _p(rg.positions),
+                                                _p(rg.row_entry), _p(page_indptr), _p(page_ids), _p(cache), page_stride, k_off,
+                                                v_off, page_size, _p(q), proj.shape[0], _dt(proj), _stream()), "qk_norm_rope_paged")
+    return q
+
+
+def paged_attention(q, cache, page_stride, k_off, v_off, page_size, rg, page_indptr, page_ids, kv_heads, vdim, scale, factor=1.0):
+    T, H, dim = q.shape
+    out = torch.empty((T, H * vdim), dtype=cache.dtype, device=q.device)
+    t = attention_tiles(rg.lens, H // kv_heads, q.device)
+    _chk(ffi.lib().pegainfer_paged_attention(_p(q), _p(cache), page_stride, k_off, v_off, page_size, _p(rg.positions),
+                                             _p(rg.row_entry), _p(page_indptr), _p(page_ids), H, kv_heads, dim, vdim,
+                                             float(scale), float(factor), _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), t[0].numel(),
+                                             _p(out), out.stride(0), _dt(cache), _stream()), "paged_attention")
     return out
