@@ -221,15 +221,16 @@ pegainfer_status_t pegainfer_head_rms_gate(const float* o, const void* w, int32_
  * pegainfer_qk_norm_rope_paged: per row from `proj` (dtype): q heads at q_off, k heads at k_off, v heads at v_off.
  *   q, k -> RMS norm over dim (eps) * q_norm / k_norm ([dim], plain weight), then neighbours (2i, 2i + 1) of the first
  *   rot_dims values rotated by position * inv_freq[i] (fp32 angles); k and v go to the cache entry of (request, position),
- *   q to q_out (fp32 [rows][heads][dim]). */
+ *   q to q_out (fp32 [rows][heads][dim]) or, when q_out_stored is given, to that buffer in dtype instead (the form the
+ *   matrix-core attention kernels of pegainfer_kernels.h read). */
 pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_stride, int64_t q_off, int64_t k_off,
                                                 int64_t v_off, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
                                                 const void* q_norm, const void* k_norm, float eps, const float* inv_freq,
                                                 int32_t rot_dims, const int32_t* positions, const int32_t* row_entry,
                                                 const int32_t* page_indptr, const int32_t* page_ids, void* cache,
                                                 int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
-                                                int32_t page_size, float* q_out, int32_t n_rows, int32_t dtype,
-                                                pegainfer_stream_t stream);
+                                                int32_t page_size, float* q_out, void* q_out_stored, int32_t n_rows,
+                                                int32_t dtype, pegainfer_stream_t stream);
 /* Causal softmax attention, scores and weights in fp32:  out[row, h, :] = factor * sum_{j <= position} softmax_j(q . k_j * scale) v_j.
  * The rows are cut by the caller into tiles that stay inside one entry: tile i covers rows tile_row0[i] .. + tile_ntok[i] - 1
  * and, of each key/value group's query heads, tile_qh0[i] .. + tile_nqh[i] - 1, with ntok * nqh <= 16.  dim, vdim <= 256.
@@ -241,6 +242,9 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                              float factor, const int32_t* tile_row0, const int32_t* tile_ntok,
                                              const int32_t* tile_qh0, const int32_t* tile_nqh, int32_t n_tiles, void* out,
                                              int64_t out_stride, int32_t dtype, pegainfer_stream_t stream);
+/* out[row, :cols] = in[row, :cols] * factor; rows of in / out at their own strides (elements of dtype) */
+pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,
+                                        int32_t rows, float factor, int32_t dtype, pegainfer_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -9,6 +9,8 @@
 //                              columns lane, lane + 64, ... for the output; running maximum / sum per row
 // Keys are always visited in tiles of 64 from position 0, whatever the step's shape, so a row's arithmetic does not depend on
 // how its prompt was cut or on what else runs in the step.
+#include <algorithm>
+
 #include "common.h"
 #include "typed.h"
 #include "pegainfer_kernels_blocks.h"
@@ -21,7 +23,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
     const A* __restrict__ q_norm, const A* __restrict__ k_norm, float eps, const float* __restrict__ inv_freq, int rot_dims,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_entry, const int32_t* __restrict__ page_indptr,
     const int32_t* __restrict__ page_ids, A* __restrict__ cache, int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
-    int page_size, float* __restrict__ q_out) {
+    int page_size, float* __restrict__ q_out, A* __restrict__ q_out_stored) {
   extern __shared__ float sm[];   // [4 waves][dim]
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int pos = positions[row], e = row_entry[row];
@@ -50,9 +52,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_paged_kernel(
         const float c = cosf(ang), s = sinf(ang);
         out = (i & 1) ? buf[i] * c + buf[i - 1] * s : buf[i] * c - buf[i + 1] * s;
       }
-      if (is_q)
-        q_out[((int64_t)row * H + hh) * dim + i] = out;
-      else
+      if (is_q) {
+        if (q_out_stored) st(q_out_stored + ((int64_t)row * H + hh) * dim + i, out);
+        else q_out[((int64_t)row * H + hh) * dim + i] = out;
+      } else
         st(cache + page * page_stride + k_cache_off + ((int64_t)slot * G + (hh - H)) * dim + i, out);
     }
     __builtin_amdgcn_wave_barrier();
@@ -160,6 +163,15 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   }
 }
 
+// out[row, :cols] = in[row, :cols] * factor, rows of either side at their own stride
+template <typename A>
+__global__ __launch_bounds__(256) void scale_rows_kernel(const A* __restrict__ in, int64_t in_stride, A* __restrict__ out,
+                                                         int64_t out_stride, int cols, float factor) {
+  const int row = blockIdx.x;
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < cols; i += gridDim.y * 256)
+    st(out + (int64_t)row * out_stride + i, ld(in + (int64_t)row * in_stride + i) * factor);
+}
+
 }  // namespace pk
 
 extern "C" {
@@ -173,8 +185,8 @@ pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_s
                                                 int32_t rot_dims, const int32_t* positions, const int32_t* row_entry,
                                                 const int32_t* page_indptr, const int32_t* page_ids, void* cache,
                                                 int64_t page_stride, int64_t k_cache_off, int64_t v_cache_off,
-                                                int32_t page_size, float* q_out, int32_t n_rows, int32_t dtype,
-                                                pegainfer_stream_t stream) {
+                                                int32_t page_size, float* q_out, void* q_out_stored, int32_t n_rows,
+                                                int32_t dtype, pegainfer_stream_t stream) {
   if (n_rows <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1) || page_size <= 0)
     return PK_BAD;
@@ -183,7 +195,8 @@ pegainfer_status_t pegainfer_qk_norm_rope_paged(const void* proj, int64_t proj_s
         qk_norm_rope_paged_kernel<A><<<n_rows, 256, (size_t)4 * dim * sizeof(float), as_stream(stream)>>>(
             static_cast<const A*>(proj), proj_stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim,
             static_cast<const A*>(q_norm), static_cast<const A*>(k_norm), eps, inv_freq, rot_dims, positions, row_entry,
-            page_indptr, page_ids, static_cast<A*>(cache), page_stride, k_cache_off, v_cache_off, page_size, q_out);
+            page_indptr, page_ids, static_cast<A*>(cache), page_stride, k_cache_off, v_cache_off, page_size, q_out,
+            static_cast<A*>(q_out_stored));
       }))
     return PK_BAD;
   return (pegainfer_status_t)hipGetLastError();
@@ -217,6 +230,19 @@ pegainfer_status_t pegainfer_paged_attention(const float* q, const void* cache, 
                                                  static_cast<A*>(out), out_stride);
   });
   return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+}
+
+pegainfer_status_t pegainfer_scale_rows(const void* in, int64_t in_stride, void* out, int64_t out_stride, int32_t cols,
+                                        int32_t rows, float factor, int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  const dim3 grid(rows, std::min(8, ceil_div(cols, 256)));
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        scale_rows_kernel<A><<<grid, 256, 0, as_stream(stream)>>>(static_cast<const A*>(in), in_stride, static_cast<A*>(out),
+                                                                  out_stride, cols, factor);
+      }))
+    return PK_BAD;
+  return (pegainfer_status_t)hipGetLastError();
 }
 
 }  // extern "C"

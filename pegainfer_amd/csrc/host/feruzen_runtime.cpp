@@ -99,6 +99,7 @@ struct LayerCfg {
   int64_t st_canon = 0, st_conv = 0, st_mem = 0;
   int64_t k_off = 0, v_off = 0;
   int tile_set = -1;
+  int fast_hd = 0;   // 128 / 256: the matrix-core attention kernels of pegainfer_kernels.h fit this layer (bf16, dim == vdim)
 };
 struct LayerW {
   void *norm1 = nullptr, *norm2 = nullptr, *canon = nullptr, *dwa = nullptr, *proj = nullptr, *o = nullptr;
@@ -130,11 +131,13 @@ struct Model {
   std::vector<KvState> requests;
   pq::StateLayout state_layout;
   float* state = nullptr;
-  std::vector<int> tile_groups;   // distinct query-heads-per-kv-head values of the attention layers
+  struct TileSet { int per = 1, fast_hd = 0, heads = 0, kv = 0; };
+  std::vector<TileSet> tile_sets;   // distinct (query heads per kv head, attention form) of the attention layers
   // step buffers
   size_t cap_rows = 0, cap_want = 0, cap_meta = 0;
   std::vector<void*> step_owned, want_owned;
   float *x = nullptr, *xs = nullptr, *qkv32 = nullptr, *q32 = nullptr, *o32 = nullptr, *ypairs = nullptr, *route_w = nullptr;
+  void *q16 = nullptr, *attn16 = nullptr;   // stored-type queries and contiguous output of the matrix-core attention
   void *hb = nullptr, *xb = nullptr, *proj = nullptr, *mix = nullptr, *y = nullptr, *gu = nullptr, *act = nullptr, *ys = nullptr,
        *gu_e = nullptr, *act_e = nullptr;
   int32_t *route_e = nullptr, *pos_pair = nullptr, *pos_row = nullptr, *tiles = nullptr;
@@ -260,10 +263,10 @@ struct Model {
         c.k_off = off;
         c.v_off = off + (int64_t)kPageSize * a.kv * a.dim;
         off = c.v_off + (int64_t)kPageSize * a.kv * a.vdim;
-        const int per = a.heads / a.kv;
-        auto it = std::find(tile_groups.begin(), tile_groups.end(), per);
-        c.tile_set = (int)(it - tile_groups.begin());
-        if (it == tile_groups.end()) tile_groups.push_back(per);
+        // matrix-core attention (the kernels Qwen3 / Qwen3.5 run): bf16, equal key and value size 128 or 256, 16-byte
+        // aligned cache parts; page_stride's own alignment is checked once all layers are known
+        if (dtype == PEGAINFER_DTYPE_BF16 && a.dim == a.vdim && (a.dim == 128 || a.dim == 256) && c.k_off % 8 == 0 && c.v_off % 8 == 0)
+          c.fast_hd = a.dim;
       } else {
         return set_error("config: layer " + li + " has an unknown mixer type");
       }
@@ -293,6 +296,17 @@ struct Model {
       layers.push_back(c);
     }
     page_stride = std::max<int64_t>(off, 1);
+    for (auto& c : layers) {
+      if (c.type != kParallel) continue;
+      if (page_stride % 8) c.fast_hd = 0;
+      const int per = c.at.heads / c.at.kv;
+      size_t k = 0;
+      while (k < tile_sets.size() && !(tile_sets[k].per == per && tile_sets[k].fast_hd == c.fast_hd &&
+                                       (!c.fast_hd || (tile_sets[k].heads == c.at.heads && tile_sets[k].kv == c.at.kv))))
+        ++k;
+      if (k == tile_sets.size()) tile_sets.push_back({per, c.fast_hd, c.at.heads, c.at.kv});
+      c.tile_set = (int)k;
+    }
     weights.resize(layers.size());
     for (auto& c : layers) {
       mx_proj = std::max(mx_proj, c.proj_rows);
@@ -623,7 +637,8 @@ struct Model {
         dalloc(&q32, n * std::max(1, mx_q), so) || dalloc(&o32, n * std::max(1, mx_o), so) || dalloc_a(&hb, n * D, so) ||
         dalloc_a(&xb, n * D, so) || dalloc_a(&proj, n * mx_proj, so) || dalloc_a(&mix, n * mx_mix, so) || dalloc_a(&y, n * D, so) ||
         dalloc_a(&gu, n * (size_t)std::max(1, 2 * mx_ff), so) || dalloc_a(&act, n * (size_t)std::max(1, mx_ff), so) ||
-        dalloc_a(&ys, n * D, so))
+        dalloc_a(&ys, n * D, so) || dalloc_a(&q16, n * (size_t)std::max(1, mx_q), so) ||
+        dalloc_a(&attn16, n * (size_t)std::max(1, mx_q), so))
       return -1;
     if (mx_top > 0 && (dalloc(&ypairs, P * D, so) || dalloc(&route_w, P, so) || dalloc(&route_e, P, so) || dalloc(&pos_pair, P, so) ||
                        dalloc(&pos_row, P, so) || dalloc(&tiles, (size_t)3 * max_tiles + 1, so) || dalloc_a(&gu_e, n * mx_gu_e, so) ||
@@ -710,14 +725,24 @@ struct Model {
     // An attention tile is a run of token rows of one entry times a run of the query heads of one key/value head, at most
     // 16 rows in all; one set of tiles per distinct heads-per-kv-head value of the model's attention layers.
     const size_t o_tok = 0, o_pos = o_tok + T, o_ent = o_pos + T, o_row0 = o_ent + T, o_slot = o_row0 + (size_t)n + 1,
-                 o_ind = o_slot + (size_t)n, o_want = o_ind + (size_t)n + 1, o_pages = o_want + (size_t)std::max(1, W);
+                 o_ind = o_slot + (size_t)n, o_lpl = o_ind + (size_t)n + 1, o_kvlen = o_lpl + (size_t)n, o_rows = o_kvlen + (size_t)n,
+                 o_want = o_rows + 1, o_pages = o_want + (size_t)std::max(1, W);
     size_t words = o_pages + total_pages;
-    std::vector<size_t> tile_off(tile_groups.size()), tile_cnt(tile_groups.size());
-    for (size_t k = 0; k < tile_groups.size(); ++k) {
-      const int per = tile_groups[k];
+    // plain sets: [row0 | ntok | qh0 | nqh] per tile.  matrix-core sets: [request | tile of the request | 0] per tile of
+    // `cta` packed (token, query head) rows, the plan batch_prefill_paged_cuda reads
+    std::vector<size_t> tile_off(tile_sets.size()), tile_cnt(tile_sets.size());
+    std::vector<int> tile_cta(tile_sets.size(), 0);
+    for (size_t k = 0; k < tile_sets.size(); ++k) {
+      const TileSet& ts = tile_sets[k];
+      const int per = ts.per;
       size_t cnt = 0;
-      for (int i = 0; i < n; ++i)
-        cnt += per <= kAttRows ? ((size_t)lens[i] + (kAttRows / per) - 1) / (kAttRows / per) : (size_t)lens[i] * ((per + kAttRows - 1) / kAttRows);
+      if (ts.fast_hd && !plain_kernels) {
+        tile_cta[k] = batch_prefill_cta_tile_q((int)T, ts.heads, ts.kv, ts.fast_hd);
+        for (int i = 0; i < n; ++i) cnt += ((size_t)lens[i] * per + tile_cta[k] - 1) / tile_cta[k];
+      } else {
+        for (int i = 0; i < n; ++i)
+          cnt += per <= kAttRows ? ((size_t)lens[i] + (kAttRows / per) - 1) / (kAttRows / per) : (size_t)lens[i] * ((per + kAttRows - 1) / kAttRows);
+      }
       tile_off[k] = words;
       tile_cnt[k] = cnt;
       words += 4 * cnt;
@@ -742,6 +767,9 @@ struct Model {
         mh[o_row0 + i] = (int32_t)t;
         mh[o_slot + i] = ids[i];
         mh[o_ind + i] = (int32_t)pg;
+        const int kv_len = st.seq_len + lens[i];
+        mh[o_kvlen + i] = kv_len;
+        mh[o_lpl + i] = kv_len % kPageSize == 0 ? kPageSize : kv_len % kPageSize;
         for (int32_t p : st.pages) mh[o_pages + pg++] = p;
         for (int k = 0; k < lens[i]; ++k, ++t) {
           mh[o_tok + t] = (int32_t)tokens[t];
@@ -751,11 +779,19 @@ struct Model {
       }
       mh[o_row0 + n] = (int32_t)t;
       mh[o_ind + n] = (int32_t)pg;
+      mh[o_rows] = (int32_t)T;
       for (int i = 0; i < W; ++i) mh[o_want + i] = want[i];
-      for (size_t k = 0; k < tile_groups.size(); ++k) {
-        const int per = tile_groups[k];
+      for (size_t k = 0; k < tile_sets.size(); ++k) {
+        const int per = tile_sets[k].per;
         int32_t *t_row0 = mh + tile_off[k], *t_ntok = t_row0 + tile_cnt[k], *t_qh0 = t_ntok + tile_cnt[k], *t_nqh = t_qh0 + tile_cnt[k];
         size_t at_ = 0, r0 = 0;
+        if (tile_cta[k]) {
+          for (int i = 0; i < n; ++i) {
+            const int tiles_i = (lens[i] * per + tile_cta[k] - 1) / tile_cta[k];
+            for (int t = 0; t < tiles_i; ++t, ++at_) { t_row0[at_] = i; t_ntok[at_] = t; t_qh0[at_] = 0; }
+          }
+          continue;
+        }
         for (int i = 0; i < n; ++i) {
           if (per <= kAttRows) {
             const int tpt = kAttRows / per;
@@ -777,7 +813,7 @@ struct Model {
     const int32_t* md = reinterpret_cast<const int32_t*>(meta_dev);
     const uint32_t* d_tok = reinterpret_cast<const uint32_t*>(md + o_tok);
     const int32_t *d_pos = md + o_pos, *d_ent = md + o_ent, *d_row0 = md + o_row0, *d_slot = md + o_slot, *d_ind = md + o_ind,
-                  *d_want = md + o_want, *d_pages = md + o_pages;
+                  *d_want = md + o_want, *d_pages = md + o_pages, *d_lpl = md + o_lpl, *d_kvlen = md + o_kvlen;
     const int Ti = (int)T;
     const int64_t slot_stride = state_layout.floats_per_slot(), xs_stride = (int64_t)cap_rows * D;
     if (tap_on) {
@@ -816,14 +852,27 @@ struct Model {
       } else {
         const AttnCfg& a = c.at;
         const MemCfg& r = c.mm;
-        FZ_K(pegainfer_qk_norm_rope_paged(proj, Mp, c.o_q, c.o_k, c.o_v, a.heads, a.kv, a.dim, a.vdim, w.q_norm, w.k_norm, eps,
-                                          w.inv_freq, a.rot_dims, d_pos, d_ent, d_ind, d_pages, cache, page_stride, c.k_off, c.v_off,
-                                          kPageSize, q32, Ti, dtype, S()));
         const size_t ts = (size_t)c.tile_set;
         const int32_t* tb = md + tile_off[ts];
-        FZ_K(pegainfer_paged_attention(q32, cache, page_stride, c.k_off, c.v_off, kPageSize, d_pos, d_ent, d_ind, d_pages, a.heads,
-                                       a.kv, a.dim, a.vdim, a.scale, c.left_scale, tb, tb + tile_cnt[ts], tb + 2 * tile_cnt[ts],
-                                       tb + 3 * tile_cnt[ts], (int)tile_cnt[ts], mix, c.mix_cols, dtype, S()));
+        const bool fast = tile_cta[ts] != 0;
+        FZ_K(pegainfer_qk_norm_rope_paged(proj, Mp, c.o_q, c.o_k, c.o_v, a.heads, a.kv, a.dim, a.vdim, w.q_norm, w.k_norm, eps,
+                                          w.inv_freq, a.rot_dims, d_pos, d_ent, d_ind, d_pages, cache, page_stride, c.k_off, c.v_off,
+                                          kPageSize, q32, fast ? q16 : nullptr, Ti, dtype, S()));
+        if (fast) {
+          // every entry is a request whose last rows are this step's: the kernel takes a row's position from the request's
+          // key count; scores and softmax state in fp32, weights rounded to bf16 where they enter the matrix cores
+          auto attn = a.dim == 256 ? batch_prefill_paged_cuda_hd256 : batch_prefill_paged_cuda;
+          if (attn(static_cast<const Half*>(q16), static_cast<Half*>(attn16), static_cast<const Half*>(cache), c.k_off, c.v_off, d_pages,
+                   d_ind, d_lpl, d_row0, tb, tb + tile_cnt[ts], tb + 2 * tile_cnt[ts], d_kvlen,
+                   reinterpret_cast<const uint32_t*>(md + o_rows), a.heads, a.kv, a.dim, kPageSize, Ti, n, (int)tile_cnt[ts],
+                   page_stride, a.scale, S()))
+            return set_error("matrix-core prefill attention failed");
+          FZ_K(pegainfer_scale_rows(attn16, (int64_t)a.heads * a.vdim, mix, c.mix_cols, a.heads * a.vdim, Ti, c.left_scale, dtype, S()));
+        } else {
+          FZ_K(pegainfer_paged_attention(q32, cache, page_stride, c.k_off, c.v_off, kPageSize, d_pos, d_ent, d_ind, d_pages, a.heads,
+                                         a.kv, a.dim, a.vdim, a.scale, c.left_scale, tb, tb + tile_cnt[ts], tb + 2 * tile_cnt[ts],
+                                         tb + 3 * tile_cnt[ts], (int)tile_cnt[ts], mix, c.mix_cols, dtype, S()));
+        }
         FZ_K(pegainfer_gated_matrix_memory(proj, Mp, c.o_rq, c.o_rk, c.o_rv, c.o_ri, c.o_rf, w.i_bias, w.f_bias, r.cap,
                                            state + c.st_mem, slot_stride, o32, r.heads, r.dim, r.vdim, d_row0, d_slot, n, dtype, S()));
         FZ_K(pegainfer_head_rms_gate(o32, w.rnorm, 1, at(proj, (size_t)c.o_rg), Mp, 1, c.right_scale, eps,

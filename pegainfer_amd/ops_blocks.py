@@ -286,7 +286,7 @@ def qk_norm_rope_paged(proj, offs, heads, kv_heads, dim, vdim, q_norm, k_norm, e
     _chk(ffi.lib().pegainfer_qk_norm_rope_paged(_p(proj), proj.stride(0), offs[0], offs[1], offs[2], heads, kv_heads, dim, vdim,
                                                 _p(q_norm), _p(k_norm), float(eps), _p(inv_freq), rot_dims, _p(rg.positions),
                                                 _p(rg.row_entry), _p(page_indptr), _p(page_ids), _p(cache), page_stride, k_off,
-                                                v_off, page_size, _p(q), proj.shape[0], _dt(proj), _stream()), "qk_norm_rope_paged")
+                                                v_off, page_size, _p(q), None, proj.shape[0], _dt(proj), _stream()), "qk_norm_rope_paged")
     return q
 
 

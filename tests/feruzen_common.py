@@ -78,6 +78,16 @@ def config_wide_heads():
     ])
 
 
+def config_real_heads():
+    """head sizes of real models (128 and 256, equal for keys and values): in bf16 the attention of these layers runs on
+    the matrix-core kernels that Qwen3 / Qwen3.5 use; the delta and memory layers get their widest register layouts"""
+    return base(64, 70, 2, 4, [
+        parallel(left(4, 2, 128, 128, 32, base=1e4), right(1, 128, 96, 12.0), 1.2, 0.8, dense(48, 2.0)),
+        delta(2, 1, 128, 128, 4, moe(16, 1.5, 4, 2, shared=(24, 1.5))),
+        parallel(left(2, 1, 256, 256, 64, base=1e6), right(2, 40, 24, 8.0), 0.9, 1.1, None),
+    ])
+
+
 def config_tiny():
     return base(48, 50, 2, 2, [delta(2, 2, 8, 8, 2, dense(32, 1.5)),
                                parallel(left(2, 1, 8, 8, 8), right(2, 8, 8, 10.0), 1.0, 1.0, moe(16, 1.5, 4, 2, shared=(16, 1.5)))])

@@ -13,7 +13,7 @@ import feruzen_common as C
 
 pytestmark = pytest.mark.gpu
 
-CONFIGS = {"a": C.config_a, "b": C.config_b, "odd": C.config_odd, "wide": C.config_wide_heads, "tiny": C.config_tiny}
+CONFIGS = {"real": C.config_real_heads, "a": C.config_a, "b": C.config_b, "odd": C.config_odd, "wide": C.config_wide_heads, "tiny": C.config_tiny}
 
 
 def check(got, ref, dtype, what=""):
@@ -34,7 +34,7 @@ def check(got, ref, dtype, what=""):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b", "odd", "wide", "tiny"])
+@pytest.mark.parametrize("name", ["a", "b", "odd", "wide", "tiny", "real"])
 def test_whole_prompt_every_position_and_every_layer(name, dtype):
     cfg = CONFIGS[name]()
     w = C.weights_for(cfg, 11, dtype)
@@ -61,7 +61,7 @@ def test_whole_prompt_every_position_and_every_layer(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "odd", "wide"])
+@pytest.mark.parametrize("name", ["a", "odd", "wide", "real"])
 def test_prefill_then_token_by_token(name, dtype):
     cfg = CONFIGS[name]()
     w = C.weights_for(cfg, 12, dtype)
@@ -134,6 +134,35 @@ def test_unequal_requests_in_one_batch_against_each_alone(dtype):
             assert np.abs(solo - g).max() <= 1e-4 * np.abs(solo).max(), q
     eng.close()
     alone.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_steps_with_real_head_sizes(dtype):
+    """portions beside single tokens where the bf16 attention runs on the matrix-core kernels: rows of several requests in
+    one launch, portions that start in the middle of a page, single decoded tokens as one-row tiles"""
+    cfg = C.config_real_heads()
+    w = C.weights_for(cfg, 31, dtype)
+    P = [C.tokens_for(cfg, n, 40 + n) for n in (90, 21, 7)]
+    refs = [C.oracle_logits(cfg, w, p) for p in P]
+    eng = C.engine_for(cfg, w, dtype, max_tokens=256)
+    ids = [eng.new_request() for _ in P]
+    plan = [[(0, 70), (1, 3)], [(0, 1), (1, 17), (2, 5)], [(0, 1), (1, 1), (2, 1)], [(0, 18), (2, 1)]]
+    at, got = [0] * 3, [[] for _ in P]
+    for stp in plan:
+        entries, want, off = [], [], 0
+        for q, n in stp:
+            entries.append((ids[q], P[q][at[q]:at[q] + n]))
+            want += list(range(off, off + n))
+            off += n
+        lg = eng.step(entries, want=want)
+        off = 0
+        for q, n in stp:
+            got[q].append(lg[off:off + n])
+            at[q] += n
+            off += n
+    for q in range(3):
+        check(np.concatenate(got[q]), refs[q][:at[q]], dtype, q)
+    eng.close()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
