@@ -160,6 +160,17 @@ struct Model {
   int tap_rows = 0;
   int mx_proj = 0, mx_mix = 0, mx_conv = 0, mx_q = 0, mx_o = 0, mx_ff = 0, mx_top = 0, mx_gu_e = 0, mx_experts = 0;
 
+  struct GraphKey {
+    int n, want; bool tokens, plain;
+    bool operator==(const GraphKey& o) const { return n == o.n && want == o.want && tokens == o.tokens && plain == o.plain; }
+  };
+  std::vector<std::pair<GraphKey, hipGraphExec_t>> graphs;   // captured decode steps, one per shape
+  bool graphs_on = [] { const char* e = getenv("PEGAINFER_FERUZEN_GRAPH"); return !(e && e[0] == '0'); }();
+  void drop_graphs() {   // the buffers a graph was recorded over are about to move
+    for (auto& g : graphs) (void)hipGraphExecDestroy(g.second);
+    graphs.clear();
+  }
+
   int set_error(const std::string& e) { err = e; return -1; }
   size_t esize() const { return dtype == PEGAINFER_DTYPE_F32 ? 4 : 2; }
   pegainfer_stream_t S() const { return reinterpret_cast<pegainfer_stream_t>(stream); }
@@ -626,6 +637,7 @@ struct Model {
   int ensure_rows(size_t T) {
     if (T <= cap_rows) return 0;
     FZ_HIP(hipStreamSynchronize(stream));
+    drop_graphs();
     free_all(&step_owned);
     cap_rows = 0;
     size_t n = 64;
@@ -650,6 +662,7 @@ struct Model {
   int ensure_want(size_t n) {
     if (n <= cap_want) return 0;
     FZ_HIP(hipStreamSynchronize(stream));
+    drop_graphs();
     free_all(&want_owned);
     cap_want = 0;
     size_t c = 16;
@@ -726,8 +739,9 @@ struct Model {
     // 16 rows in all; one set of tiles per distinct heads-per-kv-head value of the model's attention layers.
     const size_t o_tok = 0, o_pos = o_tok + T, o_ent = o_pos + T, o_row0 = o_ent + T, o_slot = o_row0 + (size_t)n + 1,
                  o_ind = o_slot + (size_t)n, o_lpl = o_ind + (size_t)n + 1, o_kvlen = o_lpl + (size_t)n, o_rows = o_kvlen + (size_t)n,
-                 o_want = o_rows + 1, o_pages = o_want + (size_t)std::max(1, W);
-    size_t words = o_pages + total_pages;
+                 o_want = o_rows + 1;
+    size_t words = o_want + (size_t)std::max(1, W);   // the page lists come last: everything before them sits at offsets that
+                                                      // depend on the step's shape only, which a captured graph relies on
     // plain sets: [row0 | ntok | qh0 | nqh] per tile.  matrix-core sets: [request | tile of the request | 0] per tile of
     // `cta` packed (token, query head) rows, the plan batch_prefill_paged_cuda reads
     std::vector<size_t> tile_off(tile_sets.size()), tile_cnt(tile_sets.size());
@@ -747,6 +761,8 @@ struct Model {
       tile_cnt[k] = cnt;
       words += 4 * cnt;
     }
+    const size_t o_pages = words;
+    words += total_pages;
     if (words > cap_meta) {
       FZ_HIP(hipStreamSynchronize(stream));
       if (meta_host) (void)hipHostFree(meta_host);
@@ -758,6 +774,7 @@ struct Model {
       FZ_HIP(hipHostMalloc(reinterpret_cast<void**>(&meta_host), c * 4, hipHostMallocDefault));
       FZ_HIP(hipMalloc(reinterpret_cast<void**>(&meta_dev), c * 4));
       cap_meta = c;
+      drop_graphs();
     }
     int32_t* mh = reinterpret_cast<int32_t*>(meta_host);
     {
@@ -828,7 +845,9 @@ struct Model {
       }
       tap_rows = Ti;
     }
-    // ---- the layers
+    // ---- the layers (everything below reads the step's shape from its arguments and the step's contents from the metadata
+    //      block, so a launch sequence recorded for one decode step serves every later step of the same shape)
+    auto run_layers = [&]() -> int {
     FZ_K(pegainfer_embed_f32(embed, d_tok, xs, D, Ti, dtype, S()));
     FZ_K(pegainfer_embed_f32(embed, d_tok, x, D, Ti, dtype, S()));
     for (size_t li = 0; li < layers.size(); ++li) {
@@ -911,6 +930,32 @@ struct Model {
       }
       if (out_tokens) FZ_K(pegainfer_batched_top1(logits16, V, W, V, top1_state, tokens_d, S()));
     }
+    return 0;
+    };
+    // a step of single tokens only (decoding) is launch-bound: its launches are captured once per shape as a hipGraph and
+    // replayed; steps with prompt portions run eagerly
+    bool single = graphs_on && !tap_on;
+    for (int i = 0; i < n && single; ++i) single = lens[i] == 1;
+    if (single) {
+      const GraphKey key{n, W, out_tokens != nullptr, plain_kernels};
+      hipGraphExec_t exec = nullptr;
+      for (auto& g : graphs)
+        if (g.first == key) exec = g.second;
+      if (!exec) {
+        hipGraph_t g = nullptr;
+        FZ_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+        const int rc = run_layers();
+        const hipError_t e = hipStreamEndCapture(stream, &g);
+        if (rc) return -1;
+        if (e != hipSuccess) return set_error("graph capture failed");
+        FZ_HIP(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0));
+        FZ_HIP(hipGraphDestroy(g));
+        graphs.emplace_back(key, exec);
+      }
+      FZ_HIP(hipGraphLaunch(exec, stream));
+    } else if (run_layers()) {
+      return -1;
+    }
     last_rows = W;
     FZ_HIP(hipEventRecord(ev1, stream));
     if (W > 0 && out_logits) FZ_HIP(hipMemcpyAsync(out_logits, logits32, (size_t)W * V * 4, hipMemcpyDeviceToHost, stream));
@@ -991,6 +1036,7 @@ struct Model {
 
   ~Model() {
     if (stream) (void)hipStreamSynchronize(stream);
+    drop_graphs();
     free_all(&owned);
     free_all(&step_owned);
     free_all(&want_owned);

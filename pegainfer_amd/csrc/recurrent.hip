@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
       }
     }
     __syncthreads();
+#pragma unroll 2
     for (int tt = 0; tt < tc; ++tt) {
       const float g = s_g[tt], beta = s_b[tt], v = s_v[tt][cl];
       float kk[NS], a0 = 0.f, a1 = 0.f;
@@ -191,6 +192,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(const A* __restrict_
     }
     __syncthreads();
     if (t0 + kRecTokens < len) nxt.issue(min(kRecTokens, len - t0 - kRecTokens), tid, load(t0 + kRecTokens));
+#pragma unroll 2
     for (int tt = 0; tt < tc; ++tt) {
       const float ig = s_i[tt], fg = s_f[tt];
       const float m_new = fmaxf(fg + m, ig);

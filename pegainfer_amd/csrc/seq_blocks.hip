@@ -7,6 +7,8 @@
 //                           sum over the streams of earlier layers (depth-weighted averaging) in one pass over the row
 //   clamp_glu_rows_kernel   g = min(gate, L), u = clamp(up, -L, L):  g sigmoid(alpha g) (u + 1)
 //   head_rms_gate_kernel    per-head RMS norm of a read-out * weight * silu / sigmoid gate * constant
+#include <algorithm>
+
 #include "common.h"
 #include "typed.h"
 #include "pegainfer_kernels_blocks.h"
@@ -37,6 +39,56 @@ __global__ __launch_bounds__(256) void time_conv_kernel(const I* __restrict__ in
   st(out + (int64_t)row * out_stride + c, acc);
 }
 
+// The same convolution for taps <= KMAX with a window in registers: a thread owns one channel and walks kConvRows rows of the
+// step; while it stays inside an entry each row costs ONE load (the window slides), the taps' weights stay in registers.
+// Window and weights are right-aligned (slot KMAX - 1 = the current row) and summed oldest first, the order of the plain
+// kernel; slots beyond the taps hold weight 0 and input 0.
+constexpr int kConvRows = 32;
+template <typename I, typename W, typename O, int KMAX>
+__global__ __launch_bounds__(256) void time_conv_window_kernel(const I* __restrict__ in, int64_t in_stride,
+                                                               const W* __restrict__ w, const float* __restrict__ state,
+                                                               int64_t slot_stride, O* __restrict__ out, int64_t out_stride,
+                                                               int C, int K, int mode, int n_rows,
+                                                               const int32_t* __restrict__ row_entry,
+                                                               const int32_t* __restrict__ entry_row0,
+                                                               const int32_t* __restrict__ entry_slot) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  float wr[KMAX], win[KMAX];
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    const int t = KMAX - 1 - j;   // rows back
+    wr[j] = t < K ? ld(w + (int64_t)c * K + (K - 1 - t)) : 0.f;
+    win[j] = 0.f;
+  }
+  const int row_begin = blockIdx.x * kConvRows, row_end = min(n_rows, row_begin + kConvRows);
+  int cur_e = -1;
+  for (int row = row_begin; row < row_end; ++row) {
+    const int e = row_entry[row];
+    if (e != cur_e) {             // first row of this walk inside the entry: fill the window's past from rows or the tail
+      cur_e = e;
+      const int r0 = entry_row0[e], local = row - r0;
+      const float* tail = state + (int64_t)entry_slot[e] * slot_stride;
+#pragma unroll
+      for (int j = 0; j < KMAX - 1; ++j) {
+        const int t = KMAX - 1 - j;
+        const int src = local - t;
+        win[j + 1] = t >= K ? 0.f : src >= 0 ? ld(in + (int64_t)(r0 + src) * in_stride + c) : tail[(int64_t)(K - 1 + src) * C + c];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < KMAX - 1; ++j) win[j] = win[j + 1];
+    const float cur = ld(in + (int64_t)row * in_stride + c);
+    win[KMAX - 1] = cur;
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) acc = fmaf(wr[j], win[j], acc);
+    if (mode & 1) acc += cur;
+    if (mode & 2) acc = silu_f(acc);
+    st(out + (int64_t)row * out_stride + c, acc);
+  }
+}
+
 template <typename I>
 __global__ __launch_bounds__(256) void time_conv_commit_kernel(const I* __restrict__ in, int64_t in_stride,
                                                                float* __restrict__ state, int64_t slot_stride, int C, int K,
@@ -53,39 +105,82 @@ __global__ __launch_bounds__(256) void time_conv_commit_kernel(const I* __restri
   }
 }
 
-template <typename Y, typename A>
-__global__ __launch_bounds__(256) void group_rms_add_kernel(const float* __restrict__ x_in, const Y* __restrict__ y,
-                                                            const A* __restrict__ w, int groups, float eps,
-                                                            float* __restrict__ x_out, A* __restrict__ xb_out, int d,
-                                                            const float* __restrict__ stack, int64_t stack_stride,
-                                                            const A* __restrict__ coef, int n_mix,
-                                                            float* __restrict__ mix_out, A* __restrict__ mixb_out) {
-  extern __shared__ float inv[];   // [groups]
+// four consecutive values of a row, widened / rounded at the edges
+__device__ __forceinline__ void ld4(const float* p, float* o) { const f32x4 v = *reinterpret_cast<const f32x4*>(p); o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
+__device__ __forceinline__ void ld4(const uint16_t* p, float* o) {
+  const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+  o[0] = bf_lo(v.x); o[1] = bf_hi(v.x); o[2] = bf_lo(v.y); o[3] = bf_hi(v.y);
+}
+__device__ __forceinline__ void st4(float* p, const float* o) { *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]}; }
+__device__ __forceinline__ void st4(uint16_t* p, const float* o) { *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf2(o[0], o[1]), pack_bf2(o[2], o[3])}; }
+
+// x_in, x_out and mix_out may name the same memory (the stream is updated in place): an element is read, then written, by
+// the same thread, and nothing else of those buffers is touched.  VEC: rows and groups are multiples of four values and every
+// pointer is 16-byte aligned - four values per load.
+template <typename Y, typename A, bool VEC>
+__global__ __launch_bounds__(256) void group_rms_add_kernel(const float* x_in, const Y* __restrict__ y,
+                                                            const A* __restrict__ w, int groups, float eps, float* x_out,
+                                                            A* __restrict__ xb_out, int d, const float* __restrict__ stack,
+                                                            int64_t stack_stride, const A* __restrict__ coef, int n_mix,
+                                                            float* mix_out, A* __restrict__ mixb_out) {
+  extern __shared__ float sm[];   // [groups] inverse root mean squares, then [n_mix] coefficients
+  float* inv = sm;
+  float* cf = sm + groups;
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int gs = d / groups;
   const Y* yr = y + (int64_t)row * d;
+  for (int j = threadIdx.x; j < n_mix; j += 256) cf[j] = ld(coef + j);
   for (int g = wave; g < groups; g += 4) {
     float ss = 0.f;
-    for (int i = lane; i < gs; i += 64) {
-      const float v = ld(yr + g * gs + i);
-      ss = fmaf(v, v, ss);
+    if (VEC) {
+      for (int i = lane * 4; i < gs; i += 256) {
+        float v[4];
+        ld4(yr + g * gs + i, v);
+        ss = fmaf(v[0], v[0], ss); ss = fmaf(v[1], v[1], ss); ss = fmaf(v[2], v[2], ss); ss = fmaf(v[3], v[3], ss);
+      }
+    } else {
+      for (int i = lane; i < gs; i += 64) {
+        const float v = ld(yr + g * gs + i);
+        ss = fmaf(v, v, ss);
+      }
     }
     ss = wave_sum(ss);
     if (lane == 0) inv[g] = 1.0f / sqrtf(ss / (float)gs + eps);
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < d; i += 256) {
+  constexpr int N = VEC ? 4 : 1;
+  for (int i = threadIdx.x * N; i < d; i += 256 * N) {
     const int64_t at = (int64_t)row * d + i;
-    float r = ld(yr + i) * inv[i / gs] * ld(w + i);
-    if (x_in) r += x_in[at];
-    if (x_out) x_out[at] = r;
-    if (xb_out) st(xb_out + at, r);
+    float r[N], yv[N], wv[N], xv[N], m[N];
+    if (VEC) { ld4(yr + i, yv); ld4(w + i, wv); } else { yv[0] = ld(yr + i); wv[0] = ld(w + i); }
+    if (x_in) { if (VEC) ld4(x_in + at, xv); else xv[0] = x_in[at]; }
+    const float scale = inv[i / gs];   // VEC: a group holds whole fours
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      r[k] = yv[k] * scale * wv[k];
+      if (x_in) r[k] += xv[k];
+      m[k] = 0.f;
+    }
+    for (int j = 0; j < n_mix - 1; ++j) {
+      float sv[N];
+      if (VEC) ld4(stack + (int64_t)j * stack_stride + at, sv); else sv[0] = stack[(int64_t)j * stack_stride + at];
+#pragma unroll
+      for (int k = 0; k < N; ++k) m[k] = fmaf(cf[j], sv[k], m[k]);
+    }
     if (n_mix > 0) {
-      float m = 0.f;
-      for (int j = 0; j < n_mix - 1; ++j) m = fmaf(ld(coef + j), stack[(int64_t)j * stack_stride + at], m);
-      m = fmaf(ld(coef + n_mix - 1), r, m);
-      if (mix_out) mix_out[at] = m;
-      if (mixb_out) st(mixb_out + at, m);
+#pragma unroll
+      for (int k = 0; k < N; ++k) m[k] = fmaf(cf[n_mix - 1], r[k], m[k]);
+    }
+    if (VEC) {
+      if (x_out) st4(x_out + at, r);
+      if (xb_out) st4(xb_out + at, r);
+      if (n_mix > 0 && mix_out) st4(mix_out + at, m);
+      if (n_mix > 0 && mixb_out) st4(mixb_out + at, m);
+    } else {
+      if (x_out) x_out[at] = r[0];
+      if (xb_out) st(xb_out + at, r[0]);
+      if (n_mix > 0 && mix_out) mix_out[at] = m[0];
+      if (n_mix > 0 && mixb_out) st(mixb_out + at, m[0]);
     }
   }
 }
@@ -145,9 +240,19 @@ pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t
            using W = std::remove_pointer_t<decltype(tw)>;
            ok = by_dtype(out_dtype, [&](auto* to) {
                   using O = std::remove_pointer_t<decltype(to)>;
-                  time_conv_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
-                      static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
-                      static_cast<O*>(out), out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot);
+                  const dim3 wgrid(ceil_div(n_rows, kConvRows), ceil_div(channels, 256));
+                  if (n_rows >= 4 * kConvRows && taps <= 4)
+                    time_conv_window_kernel<I, W, O, 4><<<wgrid, 256, 0, as_stream(stream)>>>(
+                        static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot);
+                  else if (n_rows >= 4 * kConvRows && taps <= 8)
+                    time_conv_window_kernel<I, W, O, 8><<<wgrid, 256, 0, as_stream(stream)>>>(
+                        static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, n_rows, row_entry, entry_row0, entry_slot);
+                  else
+                    time_conv_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
+                        static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
+                        static_cast<O*>(out), out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot);
                 }) && ok;
          }) && ok;
   });
@@ -173,15 +278,24 @@ pegainfer_status_t pegainfer_group_rms_add(const float* x_in, const void* y, int
                                            const float* stack, int64_t stack_stride, const void* coef, int32_t n_mix,
                                            float* mix_out, void* mixb_out, pegainfer_stream_t stream) {
   if (rows <= 0) return 0;
-  if (groups < 1 || d <= 0 || d % groups || groups > 8192 || (n_mix > 0 && !coef) || (n_mix > 1 && !stack)) return PK_BAD;
+  if (groups < 1 || d <= 0 || d % groups || groups > 8192 || n_mix > 4096 || (n_mix > 0 && !coef) || (n_mix > 1 && !stack)) return PK_BAD;
   bool ok = true;
   const bool known = by_dtype(y_dtype, [&](auto* ty) {
     using Y = std::remove_pointer_t<decltype(ty)>;
     ok = by_dtype(dtype, [&](auto* ta) {
       using A = std::remove_pointer_t<decltype(ta)>;
-      group_rms_add_kernel<Y, A><<<rows, 256, (size_t)groups * sizeof(float), as_stream(stream)>>>(
-          x_in, static_cast<const Y*>(y), static_cast<const A*>(w), groups, eps, x_out, static_cast<A*>(xb_out), d, stack,
-          stack_stride, static_cast<const A*>(coef), n_mix, mix_out, static_cast<A*>(mixb_out));
+      const size_t smem = (size_t)(groups + std::max(n_mix, 0)) * sizeof(float);
+      const bool vec = d % 4 == 0 && (d / groups) % 4 == 0 && stack_stride % 4 == 0 && host_aligned16(x_in) && host_aligned16(y) &&
+                       host_aligned16(w) && host_aligned16(x_out) && host_aligned16(xb_out) && host_aligned16(stack) &&
+                       host_aligned16(mix_out) && host_aligned16(mixb_out);
+      if (vec)
+        group_rms_add_kernel<Y, A, true><<<rows, 256, smem, as_stream(stream)>>>(
+            x_in, static_cast<const Y*>(y), static_cast<const A*>(w), groups, eps, x_out, static_cast<A*>(xb_out), d, stack,
+            stack_stride, static_cast<const A*>(coef), n_mix, mix_out, static_cast<A*>(mixb_out));
+      else
+        group_rms_add_kernel<Y, A, false><<<rows, 256, smem, as_stream(stream)>>>(
+            x_in, static_cast<const Y*>(y), static_cast<const A*>(w), groups, eps, x_out, static_cast<A*>(xb_out), d, stack,
+            stack_stride, static_cast<const A*>(coef), n_mix, mix_out, static_cast<A*>(mixb_out));
     });
   });
   return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;

@@ -65,11 +65,36 @@ def test_time_convolution_carries_its_tail_through_portions_and_slots(dtype, tap
     close(out, Fn.silu(R.tconv(seqs[0].double(), w.double())), "float32", tol32=1e-6)
 
 
+@pytest.mark.parametrize("taps", [1, 3, 4, 7, 8, 9])
+def test_time_convolution_over_long_portions(taps):
+    """steps of a few hundred rows take the form with a sliding window in registers (up to 8 taps): entries that begin in the
+    middle of a thread's walk, a tail carried into the second step, channels beyond a whole workgroup"""
+    g = torch.Generator().manual_seed(taps)
+    Cn = 300
+    w = C.bf16_round(torch.randn(Cn, taps, generator=g))
+    seqs = [C.bf16_round(torch.randn(n, Cn, generator=g)) for n in (333, 250, 40)]
+    state = torch.zeros(3, max(taps - 1, 1), Cn, device="cuda")
+    at, got = [0, 0, 0], [[], [], []]
+    for stp in [[(0, 199), (1, 101), (2, 3)], [(2, 37), (0, 134), (1, 149)]]:
+        x = torch.cat([seqs[q][at[q]:at[q] + n] for q, n in stp])
+        rg = B().Ragged([n for _, n in stp], slots=[q for q, _ in stp])
+        out = B().time_conv(dev(x, "bfloat16"), dev(w, "bfloat16"), state if taps > 1 else state[:, :0], rg, silu=True,
+                            out_dtype=torch.float32)
+        off = 0
+        for q, n in stp:
+            got[q].append(out[off:off + n].cpu())
+            at[q] += n
+            off += n
+    for q in range(3):
+        close(torch.cat(got[q]), Fn.silu(R.tconv(seqs[q].double(), w.double())), "float32", tol32=2e-6)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mult", [1, 4])        # 4: rows and groups of whole fours take the vector form
 @pytest.mark.parametrize("groups", [1, 3, 7])
-def test_grouped_output_norm_residual_and_depth_sum(dtype, groups):
+def test_grouped_output_norm_residual_and_depth_sum(dtype, groups, mult):
     g = torch.Generator().manual_seed(groups)
-    d, rows = 42 * groups // math.gcd(42, groups), 9
+    d, rows = mult * 42 * groups // math.gcd(42, groups), 9
     y, w = C.bf16_round(torch.randn(rows, d, generator=g) * 3), C.bf16_round(1 + 0.3 * torch.randn(d, generator=g))
     x = torch.randn(rows, d, generator=g)
     stack = torch.randn(3, rows, d, generator=g)
