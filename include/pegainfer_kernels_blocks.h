@@ -186,14 +186,15 @@ pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float
 /* ---- recurrent matrix memories (state per (slot, head): S [dim][vdim] fp32, row-major) ----
  * Gated delta rule.  Per row, from qkv (fp32 [rows][qkv_stride]: q heads at 0, k heads at kv_heads * dim, v heads at
  * 2 * kv_heads * dim) and the projection row `proj` (dtype; beta logits at b_off, decay inputs at a_off, one per head):
- *   q, k -> x / sqrt(sum(x^2) + 1e-6) per head (q also * dim^-1/2);  beta = sigmoid(b);  g = exp(-exp(A_log) * softplus(a + dt_bias))
+ *   q, k -> x / sqrt(sum(x^2) + 1e-6) per head (q also * dim^-1/2), IN PLACE in qkv;
+ *   beta = sigmoid(b);  g = exp(-exp(A_log) * softplus(a + dt_bias))           -> gates (fp32 scratch [rows][2 * heads])
  *   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          head h reads q / k head h / (heads / kv_heads)
- * o: fp32 [rows][heads * vdim].  dim <= 256. */
-pegainfer_status_t pegainfer_delta_rule(const float* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
-                                        int64_t b_off, int64_t a_off, const void* A_log, const void* dt_bias, float* state,
+ * o: fp32 [rows][heads * vdim].  dim <= 256.  Two launches: a prep over all rows, then the recurrence per (entry, head). */
+pegainfer_status_t pegainfer_delta_rule(float* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride, int64_t b_off,
+                                        int64_t a_off, const void* A_log, const void* dt_bias, float* gates, float* state,
                                         int64_t slot_stride, float* o, int32_t heads, int32_t kv_heads, int32_t dim,
-                                        int32_t vdim, const int32_t* entry_row0, const int32_t* entry_slot, int32_t n_entries,
-                                        int32_t dtype, pegainfer_stream_t stream);
+                                        int32_t vdim, int32_t n_rows, const int32_t* entry_row0, const int32_t* entry_slot,
+                                        int32_t n_entries, int32_t dtype, pegainfer_stream_t stream);
 /* Exponentially gated matrix memory with a running maximum (state per (slot, head): S [dim][vdim], n [dim], m; the slot's
  * region is [S of all heads | n of all heads | m of all heads]).  Per row from `proj` (dtype): q at q_off, k at k_off
  * (heads x dim), v at v_off (heads x vdim), gate inputs at i_off / f_off (one per head), biases i_bias / f_bias:

@@ -136,6 +136,8 @@ struct Model {
   // step buffers
   size_t cap_rows = 0, cap_want = 0, cap_meta = 0;
   std::vector<void*> step_owned, want_owned;
+  float *gates32 = nullptr;
+  int mx_dheads = 0;
   float *x = nullptr, *xs = nullptr, *qkv32 = nullptr, *q32 = nullptr, *o32 = nullptr, *ypairs = nullptr, *route_w = nullptr;
   void *q16 = nullptr, *attn16 = nullptr;   // stored-type queries and contiguous output of the matrix-core attention
   void *hb = nullptr, *xb = nullptr, *proj = nullptr, *mix = nullptr, *y = nullptr, *gu = nullptr, *act = nullptr, *ys = nullptr,
@@ -324,6 +326,7 @@ struct Model {
       mx_mix = std::max(mx_mix, c.mix_cols);
       mx_conv = std::max(mx_conv, c.conv_ch);
       if (c.type == kDelta) mx_o = std::max(mx_o, c.dl.heads * c.dl.vdim);
+      if (c.type == kDelta) mx_dheads = std::max(mx_dheads, c.dl.heads);
       if (c.type == kParallel) {
         mx_q = std::max(mx_q, c.at.heads * c.at.dim);
         mx_o = std::max(mx_o, c.mm.heads * c.mm.vdim);
@@ -646,7 +649,7 @@ struct Model {
     const size_t P = n * (size_t)std::max(1, mx_top);
     max_tiles = (int)((P + 63) / 64) + std::max(1, mx_experts);
     if (dalloc(&x, n * D, so) || dalloc(&xs, (layers.size() + 1) * n * D, so) || dalloc(&qkv32, n * std::max(1, mx_conv), so) ||
-        dalloc(&q32, n * std::max(1, mx_q), so) || dalloc(&o32, n * std::max(1, mx_o), so) || dalloc_a(&hb, n * D, so) ||
+        dalloc(&q32, n * std::max(1, mx_q), so) || dalloc(&gates32, n * (size_t)std::max(1, 2 * mx_dheads), so) || dalloc(&o32, n * std::max(1, mx_o), so) || dalloc_a(&hb, n * D, so) ||
         dalloc_a(&xb, n * D, so) || dalloc_a(&proj, n * mx_proj, so) || dalloc_a(&mix, n * mx_mix, so) || dalloc_a(&y, n * D, so) ||
         dalloc_a(&gu, n * (size_t)std::max(1, 2 * mx_ff), so) || dalloc_a(&act, n * (size_t)std::max(1, mx_ff), so) ||
         dalloc_a(&ys, n * D, so) || dalloc_a(&q16, n * (size_t)std::max(1, mx_q), so) ||
@@ -864,8 +867,8 @@ struct Model {
         FZ_K(pegainfer_time_conv(proj, dtype, Mp, w.conv, dtype, state + c.st_conv, slot_stride, qkv32, PEGAINFER_DTYPE_F32,
                                  c.conv_ch, c.conv_ch, d.taps, 2, d_ent, d_row0, d_slot, Ti, S()));
         FZ_K(pegainfer_time_conv_commit(proj, dtype, Mp, state + c.st_conv, slot_stride, c.conv_ch, d.taps, d_row0, d_slot, n, S()));
-        FZ_K(pegainfer_delta_rule(qkv32, c.conv_ch, proj, Mp, c.o_b, c.o_a, w.A_log, w.dt_bias, state + c.st_mem, slot_stride, o32,
-                                  d.heads, d.kv, d.dim, d.vdim, d_row0, d_slot, n, dtype, S()));
+        FZ_K(pegainfer_delta_rule(qkv32, c.conv_ch, proj, Mp, c.o_b, c.o_a, w.A_log, w.dt_bias, gates32, state + c.st_mem, slot_stride,
+                                  o32, d.heads, d.kv, d.dim, d.vdim, Ti, d_row0, d_slot, n, dtype, S()));
         FZ_K(pegainfer_head_rms_gate(o32, w.onorm, 0, at(proj, (size_t)c.o_g), Mp, 0, 1.0f, eps, mix, c.mix_cols, d.heads, d.vdim,
                                      Ti, dtype, S()));
       } else {

@@ -234,11 +234,14 @@ def route_combine_add(y_pairs, weight, add, out_dtype):
 
 def delta_rule(qkv_f32, proj, b_off, a_off, A_log, dt_bias, state, heads, kv_heads, dim, vdim, rg):
     """qkv fp32 [rows, 2 kv dim + heads vdim] (after convolution and silu), proj [rows, *] with the beta / decay inputs;
-    state fp32 [slots, heads, dim, vdim] is updated in place; returns o fp32 [rows, heads * vdim]"""
+    state fp32 [slots, heads, dim, vdim] is updated in place, and so are the q / k parts of qkv (made unit vectors);
+    returns o fp32 [rows, heads * vdim]"""
     o = torch.empty((qkv_f32.shape[0], heads * vdim), dtype=torch.float32, device=proj.device)
+    gates = torch.empty((qkv_f32.shape[0], 2 * heads), dtype=torch.float32, device=proj.device)
     _chk(ffi.lib().pegainfer_delta_rule(_p(qkv_f32), qkv_f32.stride(0), _p(proj), proj.stride(0), b_off, a_off, _p(A_log),
-                                        _p(dt_bias), _p(state), state.stride(0), _p(o), heads, kv_heads, dim, vdim,
-                                        _p(rg.entry_row0), _p(rg.entry_slot), rg.n, _dt(proj), _stream()), "delta_rule")
+                                        _p(dt_bias), _p(gates), _p(state), state.stride(0), _p(o), heads, kv_heads, dim, vdim,
+                                        qkv_f32.shape[0], _p(rg.entry_row0), _p(rg.entry_slot), rg.n, _dt(proj), _stream()),
+         "delta_rule")
     return o
 
 
