@@ -115,14 +115,18 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     const int tc = min(kRecTokens, len - t0);
     __syncthreads();
     nxt.land(tid, s_q, s_k, s_v);
-    if (tid < tc) {
-      s_g[tid] = gates[(int64_t)(row0 + t0 + tid) * 2 * H + h];
-      s_b[tid] = gates[(int64_t)(row0 + t0 + tid) * 2 * H + H + h];
+    if (tid < kRecTokens) {   // rows past the entry's end: g = 1, beta = 0, zero key - a step that leaves S as it is
+      s_g[tid] = tid < tc ? gates[(int64_t)(row0 + t0 + tid) * 2 * H + h] : 1.f;
+      s_b[tid] = tid < tc ? gates[(int64_t)(row0 + t0 + tid) * 2 * H + H + h] : 0.f;
     }
     __syncthreads();
     if (t0 + kRecTokens < len) fetch(t0 + kRecTokens);
     float okeep = 0.f;
-    for (int tt = 0; tt < tc; ++tt) {
+    // two tokens per trip: the second token's first product starts while the first token's read-out is still being summed
+    for (int t2 = 0; t2 < tc; t2 += 2) {
+#pragma unroll
+     for (int uu = 0; uu < 2; ++uu) {
+      const int tt = t2 + uu;
       const float g = s_g[tt], beta = s_b[tt], v = s_v[tt][cl];
       float kk[NS], a0 = 0.f, a1 = 0.f;
 #pragma unroll
@@ -141,6 +145,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
       }
       const float oa = row16_sum(o0 + o1);
       okeep = tt == r ? oa : okeep;      // lane r of the column keeps token r of the round
+     }
     }
     if (r < tc && col < vdim) o[(int64_t)(row0 + t0 + r) * ((int64_t)H * vdim) + (int64_t)h * vdim + col] = okeep;
   }
@@ -208,16 +213,22 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(const A* __restrict_
       }
     }
     __syncthreads();
-    if (tid < tc) {                 // ... and the exponentials it feeds are computed side by side
-      const float mp = s_m[tid], mn = s_m[tid + 1];
-      s_a[tid] = expf(s_f[tid] + mp - mn);
-      s_b[tid] = expf(s_i[tid] - mn);
-      s_em[tid] = expf(-mn);
+    if (tid < kRecTokens) {         // ... and the exponentials it feeds are computed side by side
+      const bool live = tid < tc;   // rows past the entry's end: a = 1, b = 0 - a step that leaves S and n as they are
+      const float mp = live ? s_m[tid] : 0.f, mn = live ? s_m[tid + 1] : 0.f;
+      s_a[tid] = live ? expf(s_f[tid] + mp - mn) : 1.f;
+      s_b[tid] = live ? expf(s_i[tid] - mn) : 0.f;
+      s_em[tid] = live ? expf(-mn) : 1.f;
     }
     __syncthreads();
     if (tid == 0) s_m[0] = s_m[tc];
     float okeep = 0.f;
-    for (int tt = 0; tt < tc; ++tt) {
+    // no token waits for the sums of the one before it here (only S and n carry over): four tokens per trip, their sums and
+    // quotients in flight together
+    for (int t4 = 0; t4 < tc; t4 += 4) {
+#pragma unroll
+     for (int uu = 0; uu < 4; ++uu) {
+      const int tt = t4 + uu;
       const float a = s_a[tt], b = s_b[tt];
       const float bv = b * s_v[tt][cl];
       float num0 = 0.f, num1 = 0.f, nq0 = 0.f, nq1 = 0.f;
@@ -232,6 +243,7 @@ __global__ __launch_bounds__(256) void matrix_memory_kernel(const A* __restrict_
       const float num = row16_sum(num0 + num1), nq = row16_sum(nq0 + nq1);
       const float den = fmaxf(fabsf(nq), s_em[tt]) + 1e-6f;
       okeep = tt == r ? num / den : okeep;
+     }
     }
     if (r < tc && col < vdim) o[(int64_t)(row0 + t0 + r) * ((int64_t)H * vdim) + (int64_t)h * vdim + col] = okeep;
   }
