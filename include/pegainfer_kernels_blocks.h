@@ -155,6 +155,11 @@ pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t
                                        int64_t out_row_stride, int32_t channels, int32_t taps, int32_t mode,
                                        const int32_t* row_entry, const int32_t* entry_row0, const int32_t* entry_slot,
                                        int32_t n_rows, pegainfer_stream_t stream);
+/* both in one launch for a step in which every entry brings exactly one row (row e belongs to entry e): decoding */
+pegainfer_status_t pegainfer_time_conv_step(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
+                                            float* state, int64_t slot_stride, void* out, int32_t out_dtype, int64_t out_row_stride,
+                                            int32_t channels, int32_t taps, int32_t mode, const int32_t* entry_slot,
+                                            int32_t n_entries, pegainfer_stream_t stream);
 pegainfer_status_t pegainfer_time_conv_commit(const void* in, int32_t in_dtype, int64_t in_row_stride, float* state,
                                               int64_t slot_stride, int32_t channels, int32_t taps, const int32_t* entry_row0,
                                               const int32_t* entry_slot, int32_t n_entries, pegainfer_stream_t stream);

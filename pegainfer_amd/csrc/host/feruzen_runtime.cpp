@@ -850,6 +850,8 @@ struct Model {
     }
     // ---- the layers (everything below reads the step's shape from its arguments and the step's contents from the metadata
     //      block, so a launch sequence recorded for one decode step serves every later step of the same shape)
+    bool single = true;   // every entry brings one token: decoding
+    for (int i = 0; i < n && single; ++i) single = lens[i] == 1;
     auto run_layers = [&]() -> int {
     FZ_K(pegainfer_embed_f32(embed, d_tok, xs, D, Ti, dtype, S()));
     FZ_K(pegainfer_embed_f32(embed, d_tok, x, D, Ti, dtype, S()));
@@ -858,15 +860,25 @@ struct Model {
       const LayerW& w = weights[li];
       const int Mp = c.proj_rows;
       // input convolution: hb = x + conv(x), then the tail moves on
-      FZ_K(pegainfer_time_conv(x, PEGAINFER_DTYPE_F32, D, w.canon, dtype, state + c.st_canon, slot_stride, hb, dtype, D, D,
-                               canon_taps, 1, d_ent, d_row0, d_slot, Ti, S()));
-      FZ_K(pegainfer_time_conv_commit(x, PEGAINFER_DTYPE_F32, D, state + c.st_canon, slot_stride, D, canon_taps, d_row0, d_slot, n, S()));
+      if (single) {
+        FZ_K(pegainfer_time_conv_step(x, PEGAINFER_DTYPE_F32, D, w.canon, dtype, state + c.st_canon, slot_stride, hb, dtype, D, D,
+                                      canon_taps, 1, d_slot, n, S()));
+      } else {
+        FZ_K(pegainfer_time_conv(x, PEGAINFER_DTYPE_F32, D, w.canon, dtype, state + c.st_canon, slot_stride, hb, dtype, D, D,
+                                 canon_taps, 1, d_ent, d_row0, d_slot, Ti, S()));
+        FZ_K(pegainfer_time_conv_commit(x, PEGAINFER_DTYPE_F32, D, state + c.st_canon, slot_stride, D, canon_taps, d_row0, d_slot, n, S()));
+      }
       if (linear(w.proj, hb, proj, Mp, Ti, D)) return -1;
       if (c.type == kDelta) {
         const DeltaCfg& d = c.dl;
-        FZ_K(pegainfer_time_conv(proj, dtype, Mp, w.conv, dtype, state + c.st_conv, slot_stride, qkv32, PEGAINFER_DTYPE_F32,
-                                 c.conv_ch, c.conv_ch, d.taps, 2, d_ent, d_row0, d_slot, Ti, S()));
-        FZ_K(pegainfer_time_conv_commit(proj, dtype, Mp, state + c.st_conv, slot_stride, c.conv_ch, d.taps, d_row0, d_slot, n, S()));
+        if (single) {
+          FZ_K(pegainfer_time_conv_step(proj, dtype, Mp, w.conv, dtype, state + c.st_conv, slot_stride, qkv32, PEGAINFER_DTYPE_F32,
+                                        c.conv_ch, c.conv_ch, d.taps, 2, d_slot, n, S()));
+        } else {
+          FZ_K(pegainfer_time_conv(proj, dtype, Mp, w.conv, dtype, state + c.st_conv, slot_stride, qkv32, PEGAINFER_DTYPE_F32,
+                                   c.conv_ch, c.conv_ch, d.taps, 2, d_ent, d_row0, d_slot, Ti, S()));
+          FZ_K(pegainfer_time_conv_commit(proj, dtype, Mp, state + c.st_conv, slot_stride, c.conv_ch, d.taps, d_row0, d_slot, n, S()));
+        }
         FZ_K(pegainfer_delta_rule(qkv32, c.conv_ch, proj, Mp, c.o_b, c.o_a, w.A_log, w.dt_bias, gates32, state + c.st_mem, slot_stride,
                                   o32, d.heads, d.kv, d.dim, d.vdim, Ti, d_row0, d_slot, n, dtype, S()));
         FZ_K(pegainfer_head_rms_gate(o32, w.onorm, 0, at(proj, (size_t)c.o_g), Mp, 0, 1.0f, eps, mix, c.mix_cols, d.heads, d.vdim,
@@ -937,9 +949,7 @@ struct Model {
     };
     // a step of single tokens only (decoding) is launch-bound: its launches are captured once per shape as a hipGraph and
     // replayed; steps with prompt portions run eagerly
-    bool single = graphs_on && !tap_on;
-    for (int i = 0; i < n && single; ++i) single = lens[i] == 1;
-    if (single) {
+    if (single && graphs_on && !tap_on) {
       const GraphKey key{n, W, out_tokens != nullptr, plain_kernels};
       hipGraphExec_t exec = nullptr;
       for (auto& g : graphs)

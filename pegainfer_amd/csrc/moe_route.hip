@@ -9,6 +9,8 @@
 //                   tiles the grouped GEMM walks.  The order of pairs inside an expert comes from atomics; every pair owns
 //                   its output row, so results do not depend on it.  Tiles hold <= 64 or <= 128 rows, as the GEMM form that walks them wants.
 //   combine_kernel  out[row] = sum over the row's choices, in choice order, of weight * expert output (fp32 sum).
+#include <algorithm>
+
 #include "common.h"
 #include "typed.h"
 #include "pegainfer_kernels_blocks.h"
@@ -161,7 +163,7 @@ template <typename A>
 __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restrict__ y, const float* __restrict__ w,
                                                             const A* __restrict__ add, A* __restrict__ out, int d, int top) {
   const int row = blockIdx.x;
-  for (int i = threadIdx.x; i < d; i += 256) {
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < d; i += gridDim.y * 256) {
     float a = add ? ld(add + (size_t)row * d + i) : 0.f;
     for (int c = 0; c < top; ++c) a = fmaf(w[(size_t)row * top + c], y[((size_t)row * top + c) * d + i], a);
     st(out + (size_t)row * d + i, a);
@@ -219,7 +221,9 @@ pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float
   if (rows <= 0) return 0;
   if (!by_dtype(dtype, [&](auto* t) {
         using A = std::remove_pointer_t<decltype(t)>;
-        route_combine_kernel<A><<<rows, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<const A*>(add),
+        // few rows (decoding): the row is cut over several workgroups
+        const dim3 grid(rows, rows >= 256 ? 1 : std::min(16, ceil_div(d, 256)));
+        route_combine_kernel<A><<<grid, 256, 0, as_stream(stream)>>>(y_pairs, weight, static_cast<const A*>(add),
                                                                      static_cast<A*>(out), d, top);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;

@@ -89,6 +89,31 @@ __global__ __launch_bounds__(256) void time_conv_window_kernel(const I* __restri
   }
 }
 
+// Decoding: every entry brings ONE row.  Output and the moved-on tail in one launch: a thread owns (entry, channel), reads the
+// taps - 1 carried inputs once, and writes them back shifted by one with the new input last.
+template <typename I, typename W, typename O>
+__global__ __launch_bounds__(256) void time_conv_step_kernel(const I* __restrict__ in, int64_t in_stride, const W* __restrict__ w,
+                                                             float* __restrict__ state, int64_t slot_stride, O* __restrict__ out,
+                                                             int64_t out_stride, int C, int K, int mode,
+                                                             const int32_t* __restrict__ entry_slot) {
+  const int e = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  float* tail = state + (int64_t)entry_slot[e] * slot_stride;
+  const float cur = ld(in + (int64_t)e * in_stride + c);
+  float acc = 0.f;
+  for (int j = 0; j < K - 1; ++j) {
+    const float v = tail[(int64_t)j * C + c];
+    acc = fmaf(ld(w + (int64_t)c * K + j), v, acc);
+    if (j > 0) tail[(int64_t)(j - 1) * C + c] = v;
+  }
+  acc = fmaf(ld(w + (int64_t)c * K + K - 1), cur, acc);
+  if (K > 1) tail[(int64_t)(K - 2) * C + c] = cur;
+  if (mode & 1) acc += cur;
+  if (mode & 2) acc = silu_f(acc);
+  st(out + (int64_t)e * out_stride + c, acc);
+}
+
 template <typename I>
 __global__ __launch_bounds__(256) void time_conv_commit_kernel(const I* __restrict__ in, int64_t in_stride,
                                                                float* __restrict__ state, int64_t slot_stride, int C, int K,
@@ -253,6 +278,29 @@ pegainfer_status_t pegainfer_time_conv(const void* in, int32_t in_dtype, int64_t
                     time_conv_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
                         static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
                         static_cast<O*>(out), out_row_stride, channels, taps, mode, row_entry, entry_row0, entry_slot);
+                }) && ok;
+         }) && ok;
+  });
+  return known && ok ? (pegainfer_status_t)hipGetLastError() : PK_BAD;
+}
+
+pegainfer_status_t pegainfer_time_conv_step(const void* in, int32_t in_dtype, int64_t in_row_stride, const void* w, int32_t w_dtype,
+                                            float* state, int64_t slot_stride, void* out, int32_t out_dtype, int64_t out_row_stride,
+                                            int32_t channels, int32_t taps, int32_t mode, const int32_t* entry_slot,
+                                            int32_t n_entries, pegainfer_stream_t stream) {
+  if (n_entries <= 0) return 0;
+  if (channels <= 0 || taps < 1) return PK_BAD;
+  const dim3 grid(n_entries, ceil_div(channels, 256));
+  bool ok = true;
+  const bool known = by_dtype(in_dtype, [&](auto* ti) {
+    using I = std::remove_pointer_t<decltype(ti)>;
+    ok = by_dtype(w_dtype, [&](auto* tw) {
+           using W = std::remove_pointer_t<decltype(tw)>;
+           ok = by_dtype(out_dtype, [&](auto* to) {
+                  using O = std::remove_pointer_t<decltype(to)>;
+                  time_conv_step_kernel<I, W, O><<<grid, 256, 0, as_stream(stream)>>>(
+                      static_cast<const I*>(in), in_row_stride, static_cast<const W*>(w), state, slot_stride,
+                      static_cast<O*>(out), out_row_stride, channels, taps, mode, entry_slot);
                 }) && ok;
          }) && ok;
   });

@@ -184,6 +184,11 @@ def time_conv(x, w, state, rg, residual=False, silu=False, out_dtype=None, chann
     out = torch.empty((x.shape[0], C), dtype=out_dtype or x.dtype, device=x.device)
     slot_stride = state.shape[1] * state.shape[2] if state.dim() == 3 else 0
     L = ffi.lib()
+    if all(n == 1 for n in rg.lens):      # decoding: output and the moved-on tail in one launch
+        _chk(L.pegainfer_time_conv_step(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(state), slot_stride, _p(out), _dt(out), C, C,
+                                        taps, (1 if residual else 0) | (2 if silu else 0), _p(rg.entry_slot), rg.n, _stream()),
+             "time_conv_step")
+        return out
     _chk(L.pegainfer_time_conv(_p(x), _dt(x), x.stride(0), _p(w), _dt(w), _p(state), slot_stride, _p(out), _dt(out), C, C, taps,
                                (1 if residual else 0) | (2 if silu else 0), _p(rg.row_entry), _p(rg.entry_row0),
                                _p(rg.entry_slot), x.shape[0], _stream()), "time_conv")

@@ -44,7 +44,8 @@ def test_time_convolution_carries_its_tail_through_portions_and_slots(dtype, tap
     state = torch.full((3, max(taps - 1, 1), Cn), 7.0, device="cuda")      # dirty: slots 2 and 0 are zeroed for the new requests
     state[2].zero_()
     state[0].zero_()
-    plans = [[(0, 1), (1, 2)], [(0, 2), (1, 1)], [(0, 13)], [(0, 7), (1, 6)]]    # (sequence, rows) per step; slots 2 and 0
+    plans = [[(0, 1), (1, 2)], [(0, 2), (1, 1)], [(0, 1), (1, 1)], [(0, 12)], [(0, 7), (1, 5)]]    # (sequence, rows) per step;
+    # slots 2 and 0; the third step brings one row per entry: the decode form (output and tail in one launch)
     at, got = [0, 0], [[], []]
     for stp in plans:
         x = torch.cat([seqs[q][at[q]:at[q] + n] for q, n in stp])
