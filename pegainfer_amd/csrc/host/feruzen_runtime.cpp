@@ -139,6 +139,8 @@ struct Model {
   float *gates32 = nullptr;
   int mx_dheads = 0;
   float *x = nullptr, *xs = nullptr, *qkv32 = nullptr, *q32 = nullptr, *o32 = nullptr, *ypairs = nullptr, *route_w = nullptr;
+  Half* split_tmp_v = nullptr;   // partials of the partition decode attention
+  float* split_tmp_s = nullptr;
   void *q16 = nullptr, *attn16 = nullptr;   // stored-type queries and contiguous output of the matrix-core attention
   void *hb = nullptr, *xb = nullptr, *proj = nullptr, *mix = nullptr, *y = nullptr, *gu = nullptr, *act = nullptr, *ys = nullptr,
        *gu_e = nullptr, *act_e = nullptr;
@@ -163,8 +165,8 @@ struct Model {
   int mx_proj = 0, mx_mix = 0, mx_conv = 0, mx_q = 0, mx_o = 0, mx_ff = 0, mx_top = 0, mx_gu_e = 0, mx_experts = 0;
 
   struct GraphKey {
-    int n, want; bool tokens, plain;
-    bool operator==(const GraphKey& o) const { return n == o.n && want == o.want && tokens == o.tokens && plain == o.plain; }
+    int n, want; bool tokens, plain; int split;
+    bool operator==(const GraphKey& o) const { return n == o.n && want == o.want && tokens == o.tokens && plain == o.plain && split == o.split; }
   };
   std::vector<std::pair<GraphKey, hipGraphExec_t>> graphs;   // captured decode steps, one per shape
   bool graphs_on = [] { const char* e = getenv("PEGAINFER_FERUZEN_GRAPH"); return !(e && e[0] == '0'); }();
@@ -374,6 +376,11 @@ struct Model {
     requests.assign((size_t)max_requests, KvState());
     if (dalloc_a(&cache, (size_t)num_pages * (size_t)page_stride)) return -1;
     if (dalloc(&state, (size_t)max_requests * (size_t)state_layout.floats_per_slot())) return -1;
+    bool any_fast = false;
+    for (auto& c : layers) any_fast = any_fast || c.fast_hd != 0;
+    if (any_fast && (dalloc(&split_tmp_v, (size_t)max_requests * pq::kSplitMaxChunksPerRequest * (size_t)std::max(1, mx_q)) ||
+                     dalloc(&split_tmp_s, (size_t)max_requests * pq::kSplitMaxChunksPerRequest * (size_t)std::max(1, mx_q))))
+      return -1;
     if (dalloc(&probs_scratch, (size_t)V) || dalloc(&top1_value, 1) || dalloc(&row_states, 1024 * 1024) ||
         dalloc(&valid_scratch, 1) || dalloc(&sample_out_d, 1))
       return -1;
@@ -740,6 +747,8 @@ struct Model {
     //   tokens | positions | row_entry | entry_row0 | entry_slot | page_indptr | want | page_ids | attention tile sets
     // An attention tile is a run of token rows of one entry times a run of the query heads of one key/value head, at most
     // 16 rows in all; one set of tiles per distinct heads-per-kv-head value of the model's attention layers.
+    bool single = true;   // every entry brings one token: decoding
+    for (int i = 0; i < n && single; ++i) single = lens[i] == 1;
     const size_t o_tok = 0, o_pos = o_tok + T, o_ent = o_pos + T, o_row0 = o_ent + T, o_slot = o_row0 + (size_t)n + 1,
                  o_ind = o_slot + (size_t)n, o_lpl = o_ind + (size_t)n + 1, o_kvlen = o_lpl + (size_t)n, o_rows = o_kvlen + (size_t)n,
                  o_want = o_rows + 1;
@@ -747,12 +756,28 @@ struct Model {
                                                       // depend on the step's shape only, which a captured graph relies on
     // plain sets: [row0 | ntok | qh0 | nqh] per tile.  matrix-core sets: [request | tile of the request | 0] per tile of
     // `cta` packed (token, query head) rows, the plan batch_prefill_paged_cuda reads
+    // matrix-core sets of a decoding step: the partition plan of the framework's decode attention instead (kv_pool.h
+    // make_split_plan: every request's keys cut into chunks that run as workgroups of their own, merged afterwards),
+    //   [request per slot | chunk per slot | chunk size | output indptr | zeros (n) | valid bytes per slot]
     std::vector<size_t> tile_off(tile_sets.size()), tile_cnt(tile_sets.size());
     std::vector<int> tile_cta(tile_sets.size(), 0);
+    std::vector<pq::SplitPlan> dplan(tile_sets.size());
+    int split_mask = 0;
     for (size_t k = 0; k < tile_sets.size(); ++k) {
       const TileSet& ts = tile_sets[k];
       const int per = ts.per;
       size_t cnt = 0;
+      if (ts.fast_hd && !plain_kernels && single) {
+        std::vector<int> kv_lens(n);
+        for (int i = 0; i < n; ++i) kv_lens[i] = requests[ids[i]].seq_len + 1;
+        dplan[k] = pq::make_split_plan(1, kv_lens, n, ts.kv, false);
+        if (dplan[k].use_split) split_mask |= 1 << (k & 30);
+        tile_cta[k] = -1;
+        tile_off[k] = words;
+        tile_cnt[k] = (size_t)dplan[k].slots;
+        words += 2 * tile_cnt[k] + 1 + (size_t)n + 1 + (size_t)n + (tile_cnt[k] + 3) / 4;
+        continue;
+      }
       if (ts.fast_hd && !plain_kernels) {
         tile_cta[k] = batch_prefill_cta_tile_q((int)T, ts.heads, ts.kv, ts.fast_hd);
         for (int i = 0; i < n; ++i) cnt += ((size_t)lens[i] * per + tile_cta[k] - 1) / tile_cta[k];
@@ -805,6 +830,18 @@ struct Model {
         const int per = tile_sets[k].per;
         int32_t *t_row0 = mh + tile_off[k], *t_ntok = t_row0 + tile_cnt[k], *t_qh0 = t_ntok + tile_cnt[k], *t_nqh = t_qh0 + tile_cnt[k];
         size_t at_ = 0, r0 = 0;
+        if (tile_cta[k] < 0) {
+          const pq::SplitPlan& pl = dplan[k];
+          const size_t sl = tile_cnt[k];
+          int32_t* b = mh + tile_off[k];
+          std::memcpy(b, pl.request_indices.data(), sl * 4);
+          std::memcpy(b + sl, pl.kv_tile_indices.data(), sl * 4);
+          b[2 * sl] = pl.chunk;
+          std::memcpy(b + 2 * sl + 1, pl.o_indptr.data(), (size_t)(n + 1) * 4);
+          std::memset(b + 2 * sl + 1 + n + 1, 0, (size_t)n * 4);
+          std::memcpy(b + 2 * sl + 1 + n + 1 + n, pl.valid.data(), sl);
+          continue;
+        }
         if (tile_cta[k]) {
           for (int i = 0; i < n; ++i) {
             const int tiles_i = (lens[i] * per + tile_cta[k] - 1) / tile_cta[k];
@@ -850,8 +887,6 @@ struct Model {
     }
     // ---- the layers (everything below reads the step's shape from its arguments and the step's contents from the metadata
     //      block, so a launch sequence recorded for one decode step serves every later step of the same shape)
-    bool single = true;   // every entry brings one token: decoding
-    for (int i = 0; i < n && single; ++i) single = lens[i] == 1;
     auto run_layers = [&]() -> int {
     FZ_K(pegainfer_embed_f32(embed, d_tok, xs, D, Ti, dtype, S()));
     FZ_K(pegainfer_embed_f32(embed, d_tok, x, D, Ti, dtype, S()));
@@ -888,11 +923,32 @@ struct Model {
         const MemCfg& r = c.mm;
         const size_t ts = (size_t)c.tile_set;
         const int32_t* tb = md + tile_off[ts];
-        const bool fast = tile_cta[ts] != 0;
+        const bool fast = tile_cta[ts] != 0, fast_decode = tile_cta[ts] < 0;
         FZ_K(pegainfer_qk_norm_rope_paged(proj, Mp, c.o_q, c.o_k, c.o_v, a.heads, a.kv, a.dim, a.vdim, w.q_norm, w.k_norm, eps,
                                           w.inv_freq, a.rot_dims, d_pos, d_ent, d_ind, d_pages, cache, page_stride, c.k_off, c.v_off,
                                           kPageSize, q32, fast ? q16 : nullptr, Ti, dtype, S()));
-        if (fast) {
+        if (fast_decode) {
+          // decoding: one query row per request; long contexts are cut into chunks that run side by side (partials in bf16)
+          const size_t sl = tile_cnt[ts];
+          const int32_t *sri = tb, *skt = tb + sl, *skc = tb + 2 * sl, *soi = skc + 1, *zeros = soi + n + 1;
+          const uint8_t* sva = reinterpret_cast<const uint8_t*>(zeros + n);
+          const Half *q = static_cast<const Half*>(q16), *kv = static_cast<const Half*>(cache);
+          Half* out = static_cast<Half*>(attn16);
+          int rc;
+          if (dplan[ts].use_split)
+            rc = a.dim == 256 ? pegainfer_paged_attention_decode_split_kv_hd256(q, out, kv, c.k_off, c.v_off, d_pages, d_ind, d_lpl, sri, skt, skc, soi, sva,
+                                                                                split_tmp_v, split_tmp_s, a.heads, a.kv, a.dim, kPageSize, n, (int)sl,
+                                                                                page_stride, a.scale, nullptr, S())
+                              : paged_attention_decode_split_kv_cuda(q, out, kv, c.k_off, c.v_off, d_pages, d_ind, d_lpl, sri, skt, skc, soi, sva, split_tmp_v,
+                                                                     split_tmp_s, a.heads, a.kv, a.dim, kPageSize, n, (int)sl, page_stride, a.scale, S());
+          else
+            rc = a.dim == 256 ? paged_attention_decode_cuda_hd256(q, out, kv, c.k_off, c.v_off, d_pages, d_ind, d_lpl, d_ent, zeros, d_kvlen, a.heads, a.kv,
+                                                                  a.dim, kPageSize, n, page_stride, a.scale, S())
+                              : paged_attention_decode_cuda(q, out, kv, c.k_off, c.v_off, d_pages, d_ind, d_lpl, d_ent, zeros, d_kvlen, a.heads, a.kv, a.dim,
+                                                            kPageSize, n, page_stride, a.scale, S());
+          if (rc) return set_error("matrix-core decode attention failed");
+          FZ_K(pegainfer_scale_rows(attn16, (int64_t)a.heads * a.vdim, mix, c.mix_cols, a.heads * a.vdim, Ti, c.left_scale, dtype, S()));
+        } else if (fast) {
           // every entry is a request whose last rows are this step's: the kernel takes a row's position from the request's
           // key count; scores and softmax state in fp32, weights rounded to bf16 where they enter the matrix cores
           auto attn = a.dim == 256 ? batch_prefill_paged_cuda_hd256 : batch_prefill_paged_cuda;
@@ -950,7 +1006,7 @@ struct Model {
     // a step of single tokens only (decoding) is launch-bound: its launches are captured once per shape as a hipGraph and
     // replayed; steps with prompt portions run eagerly
     if (single && graphs_on && !tap_on) {
-      const GraphKey key{n, W, out_tokens != nullptr, plain_kernels};
+      const GraphKey key{n, W, out_tokens != nullptr, plain_kernels, split_mask};
       hipGraphExec_t exec = nullptr;
       for (auto& g : graphs)
         if (g.first == key) exec = g.second;

@@ -208,6 +208,26 @@ def test_long_decoding_across_pages_and_key_tiles():
     eng.close()
 
 
+def test_long_decoding_with_real_head_sizes_cuts_the_keys():
+    """bf16, head sizes 128 / 256: single-token steps run the framework's partition decode attention, which cuts a request's
+    keys into chunks from 65 tokens on; two requests of different lengths decode side by side, across the first cut and on"""
+    cfg = C.config_real_heads()
+    w = C.weights_for(cfg, 32, "bfloat16")
+    A, B_ = C.tokens_for(cfg, 230, 50), C.tokens_for(cfg, 150, 51)
+    ra, rb = C.oracle_logits(cfg, w, A), C.oracle_logits(cfg, w, B_)
+    eng = C.engine_for(cfg, w, "bfloat16", max_tokens=512)
+    a, b = eng.new_request(), eng.new_request()
+    eng.step([(a, A[:100]), (b, B_[:20])], want=[])
+    ga, gb = [], []
+    for t in range(130):
+        lg = eng.step([(a, [A[100 + t]]), (b, [B_[20 + t]])])
+        ga.append(lg[0])
+        gb.append(lg[1])
+    check(np.stack(ga), ra[100:230], "bfloat16", "a")
+    check(np.stack(gb), rb[20:150], "bfloat16", "b")
+    eng.close()
+
+
 def test_checkpoint_folder_through_the_registry_and_trace_replay(tmp_path):
     from safetensors.torch import save_file
     from pegainfer_amd import registry
