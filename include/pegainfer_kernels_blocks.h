@@ -184,6 +184,11 @@ enum { PEGAINFER_SCORE_SIGMOID = 0, PEGAINFER_SCORE_SOFTMAX = 1 };
 pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, const void* correction, int32_t* out_expert,
                                         float* out_weight, int32_t d, int32_t experts, int32_t n_groups, int32_t keep_groups,
                                         int32_t top, int32_t rows, int32_t score_kind, int32_t dtype, pegainfer_stream_t stream);
+/* the selection alone, from router logits a GEMM has left in fp32 ([rows, experts]; correction of dtype or NULL): the few-rows
+ * GEMM streams the router once with the whole chip where one workgroup per row would read it alone (decoding) */
+pegainfer_status_t pegainfer_route_from_logits(const float* logits, const void* correction, int32_t* out_expert, float* out_weight,
+                                               int32_t experts, int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                               int32_t score_kind, int32_t dtype, pegainfer_stream_t stream);
 /* pegainfer_route_combine plus a row every token gets (a shared expert's output, [rows, d] of dtype; NULL = none) */
 pegainfer_status_t pegainfer_route_combine_add(const float* y_pairs, const float* weight, const void* add, void* out, int32_t d,
                                                int32_t top, int32_t rows, int32_t dtype, pegainfer_stream_t stream);

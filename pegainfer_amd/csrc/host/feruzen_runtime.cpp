@@ -138,7 +138,7 @@ struct Model {
   std::vector<void*> step_owned, want_owned;
   float *gates32 = nullptr;
   int mx_dheads = 0;
-  float *x = nullptr, *xs = nullptr, *qkv32 = nullptr, *q32 = nullptr, *o32 = nullptr, *ypairs = nullptr, *route_w = nullptr;
+  float *x = nullptr, *xs = nullptr, *qkv32 = nullptr, *q32 = nullptr, *o32 = nullptr, *ypairs = nullptr, *route_w = nullptr, *route_logits = nullptr;
   Half* split_tmp_v = nullptr;   // partials of the partition decode attention
   float* split_tmp_s = nullptr;
   void *q16 = nullptr, *attn16 = nullptr;   // stored-type queries and contiguous output of the matrix-core attention
@@ -662,7 +662,7 @@ struct Model {
         dalloc_a(&ys, n * D, so) || dalloc_a(&q16, n * (size_t)std::max(1, mx_q), so) ||
         dalloc_a(&attn16, n * (size_t)std::max(1, mx_q), so))
       return -1;
-    if (mx_top > 0 && (dalloc(&ypairs, P * D, so) || dalloc(&route_w, P, so) || dalloc(&route_e, P, so) || dalloc(&pos_pair, P, so) ||
+    if (mx_top > 0 && (dalloc(&ypairs, P * D, so) || dalloc(&route_w, P, so) || dalloc(&route_logits, n * (size_t)std::max(1, mx_experts), so) || dalloc(&route_e, P, so) || dalloc(&pos_pair, P, so) ||
                        dalloc(&pos_row, P, so) || dalloc(&tiles, (size_t)3 * max_tiles + 1, so) || dalloc_a(&gu_e, n * mx_gu_e, so) ||
                        dalloc_a(&act_e, n * (size_t)(mx_gu_e / 2), so)))
       return -1;
@@ -1039,7 +1039,16 @@ struct Model {
     const MlpCfg& f = c.mlp;
     const int ff = f.glu.ff, P = T * f.top;
     int32_t *t_group = tiles, *t_row0 = tiles + max_tiles, *t_rows = tiles + 2 * max_tiles, *n_tiles = tiles + 3 * max_tiles;
-    FZ_K(pegainfer_route_topk(xb, w.router, nullptr, route_e, route_w, D, f.experts, 1, 1, f.top, T, PEGAINFER_SCORE_SOFTMAX, dtype, S()));
+    {  // router logits in fp32 by a GEMM over the stored values, then softmax over all experts and the top choices per row
+      pegainfer_gemm_desc r{};
+      r.x = xb; r.w = w.router; r.y = route_logits;
+      r.x_dtype = r.w_dtype = dtype; r.y_dtype = PEGAINFER_DTYPE_F32;
+      r.m = f.experts; r.k = D; r.rows = T; r.groups = 1;
+      r.x_row_stride = D; r.w_m_stride = D; r.w_k_stride = 1; r.y_row_stride = f.experts;
+      r.plain = plain_kernels;
+      FZ_K(pegainfer_gemm_strided(&r, S()));
+      FZ_K(pegainfer_route_from_logits(route_logits, nullptr, route_e, route_w, f.experts, 1, 1, f.top, T, PEGAINFER_SCORE_SOFTMAX, dtype, S()));
+    }
     const int per_tile = dtype == PEGAINFER_DTYPE_BF16 && !plain_kernels && T > 8 && D % 8 == 0 && ff % 8 == 0 ? 128 : 64;
     FZ_K(pegainfer_route_sort(route_e, P, f.top, f.experts, pos_pair, pos_row, t_group, t_row0, t_rows, n_tiles, max_tiles, per_tile, S()));
     pegainfer_gemm_desc d{};

@@ -17,55 +17,13 @@
 
 namespace pk {
 
+// Selection on one wave from per-expert values in LDS (s: sigmoid scores, or logits when score is softmax; ch: s + correction):
+// softmax over ALL experts if asked, group scores, kept groups, then `top` wave-wide arg-max steps.  LDS accesses of one wave
+// complete in order, so no barrier is needed between its steps.
 template <typename A>
-__global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, const A* __restrict__ wr,
-                                                    const A* __restrict__ corr, int32_t* __restrict__ out_e,
-                                                    float* __restrict__ out_w, int d, int E, int G, int keep, int top,
-                                                    int score) {
-  extern __shared__ float sm[];
-  float* s = sm;            // [E] sigmoid scores
-  float* ch = sm + E;       // [E] choice scores (eligible) or -inf
-  float* gs = sm + 2 * E;   // [G] group scores
-  const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const A* x = h + (size_t)row * d;
-  const bool vec = (d & 7) == 0 && aligned16(x) && aligned16(wr);
-  // a wave takes four experts at a time (four independent weight streams in flight), waves interleaved over the groups of four
-  constexpr int EB = 4;
-  for (int e0 = wave * EB; e0 < E; e0 += 4 * EB) {
-    float a[EB] = {0.f, 0.f, 0.f, 0.f};
-    if (vec) {
-      for (int i = lane * 8; i < d; i += 512) {
-        float xv[8];
-        Vec8<A>::load(x + i, xv);
-#pragma unroll
-        for (int q = 0; q < EB; ++q) {
-          float wv[8];
-          Vec8<A>::load(wr + (size_t)min(e0 + q, E - 1) * d + i, wv);
-#pragma unroll
-          for (int k = 0; k < 8; ++k) a[q] = fmaf(xv[k], wv[k], a[q]);
-        }
-      }
-    } else {
-      for (int i = lane; i < d; i += 64) {
-        const float xv = ld(x + i);
-#pragma unroll
-        for (int q = 0; q < EB; ++q) a[q] = fmaf(xv, ld(wr + (size_t)min(e0 + q, E - 1) * d + i), a[q]);
-      }
-    }
-#pragma unroll
-    for (int q = 0; q < EB; ++q) {
-      const float z = wave_sum(a[q]);
-      const int e = e0 + q;
-      if (lane == 0 && e < E) {
-        const float sc = score == PEGAINFER_SCORE_SOFTMAX ? z : sigmoid_f(z);   // softmax: the logit for now
-        s[e] = sc;
-        ch[e] = corr ? sc + ld(corr + e) : sc;
-      }
-    }
-  }
-  __syncthreads();
-  if (wave != 0) return;
-  // ---- selection by wave 0 alone: LDS accesses of one wave complete in order, so no barrier is needed between its steps
+__device__ __forceinline__ void route_select_wave(float* s, float* ch, float* gs, const A* __restrict__ corr,
+                                                  int32_t* __restrict__ out_e, float* __restrict__ out_w, int row, int lane, int E,
+                                                  int G, int keep, int top, int score) {
   if (score == PEGAINFER_SCORE_SOFTMAX) {            // s = exp(z - max) / sum over ALL experts, then the choice scores
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -124,6 +82,79 @@ __global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, con
     }
     __builtin_amdgcn_wave_barrier();
   }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void route_kernel(const A* __restrict__ h, const A* __restrict__ wr,
+                                                    const A* __restrict__ corr, int32_t* __restrict__ out_e,
+                                                    float* __restrict__ out_w, int d, int E, int G, int keep, int top,
+                                                    int score) {
+  extern __shared__ float sm[];
+  float* s = sm;            // [E] sigmoid scores
+  float* ch = sm + E;       // [E] choice scores (eligible) or -inf
+  float* gs = sm + 2 * E;   // [G] group scores
+  const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const A* x = h + (size_t)row * d;
+  const bool vec = (d & 7) == 0 && aligned16(x) && aligned16(wr);
+  // a wave takes four experts at a time (four independent weight streams in flight), waves interleaved over the groups of four
+  constexpr int EB = 4;
+  for (int e0 = wave * EB; e0 < E; e0 += 4 * EB) {
+    float a[EB] = {0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      for (int i = lane * 8; i < d; i += 512) {
+        float xv[8];
+        Vec8<A>::load(x + i, xv);
+#pragma unroll
+        for (int q = 0; q < EB; ++q) {
+          float wv[8];
+          Vec8<A>::load(wr + (size_t)min(e0 + q, E - 1) * d + i, wv);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) a[q] = fmaf(xv[k], wv[k], a[q]);
+        }
+      }
+    } else {
+      for (int i = lane; i < d; i += 64) {
+        const float xv = ld(x + i);
+#pragma unroll
+        for (int q = 0; q < EB; ++q) a[q] = fmaf(xv, ld(wr + (size_t)min(e0 + q, E - 1) * d + i), a[q]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < EB; ++q) {
+      const float z = wave_sum(a[q]);
+      const int e = e0 + q;
+      if (lane == 0 && e < E) {
+        const float sc = score == PEGAINFER_SCORE_SOFTMAX ? z : sigmoid_f(z);   // softmax: the logit for now
+        s[e] = sc;
+        ch[e] = corr ? sc + ld(corr + e) : sc;
+      }
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  route_select_wave(s, ch, gs, corr, out_e, out_w, row, lane, E, G, keep, top, score);
+}
+
+// The same selection from router logits that a GEMM has left in fp32 ([rows][E]): a wave per row, four rows per workgroup.
+template <typename A>
+__global__ __launch_bounds__(256) void route_from_logits_kernel(const float* __restrict__ logits, const A* __restrict__ corr,
+                                                                int32_t* __restrict__ out_e, float* __restrict__ out_w, int E,
+                                                                int G, int keep, int top, int rows, int score) {
+  extern __shared__ float sm[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  float* s = sm + wave * (2 * E + G);
+  float* ch = s + E;
+  float* gs = s + 2 * E;
+  for (int e = lane; e < E; e += 64) {
+    const float z = logits[(size_t)row * E + e];
+    const float sc = score == PEGAINFER_SCORE_SOFTMAX ? z : sigmoid_f(z);
+    s[e] = sc;
+    ch[e] = corr ? sc + ld(corr + e) : sc;
+  }
+  __builtin_amdgcn_wave_barrier();
+  route_select_wave(s, ch, gs, corr, out_e, out_w, row, lane, E, G, keep, top, score);
 }
 
 __global__ __launch_bounds__(256) void route_sort_kernel(const int32_t* __restrict__ expert, int n_pairs, int top, int E,
@@ -190,6 +221,24 @@ pegainfer_status_t pegainfer_route_topk(const void* h, const void* w_router, con
         route_kernel<A><<<rows, 256, smem, as_stream(stream)>>>(static_cast<const A*>(h), static_cast<const A*>(w_router),
                                                                 static_cast<const A*>(correction), out_expert, out_weight, d,
                                                                 experts, n_groups, keep_groups, top, score_kind);
+      }))
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  return (pegainfer_status_t)hipGetLastError();
+}
+
+pegainfer_status_t pegainfer_route_from_logits(const float* logits, const void* correction, int32_t* out_expert, float* out_weight,
+                                               int32_t experts, int32_t n_groups, int32_t keep_groups, int32_t top, int32_t rows,
+                                               int32_t score_kind, int32_t dtype, pegainfer_stream_t stream) {
+  if (rows <= 0) return 0;
+  if (n_groups < 1) n_groups = 1;
+  if (experts <= 0 || experts % n_groups || top <= 0 || top > experts || keep_groups < 1 || keep_groups > n_groups ||
+      (size_t)(2 * experts + n_groups) * 16 > 60000 || (score_kind != PEGAINFER_SCORE_SIGMOID && score_kind != PEGAINFER_SCORE_SOFTMAX))
+    return (pegainfer_status_t)hipErrorInvalidValue;
+  const size_t smem = (size_t)4 * (2 * experts + n_groups) * sizeof(float);
+  if (!by_dtype(dtype, [&](auto* t) {
+        using A = std::remove_pointer_t<decltype(t)>;
+        route_from_logits_kernel<A><<<ceil_div(rows, 4), 256, smem, as_stream(stream)>>>(
+            logits, static_cast<const A*>(correction), out_expert, out_weight, experts, n_groups, keep_groups, top, rows, score_kind);
       }))
     return (pegainfer_status_t)hipErrorInvalidValue;
   return (pegainfer_status_t)hipGetLastError();

@@ -228,6 +228,16 @@ def route_topk(h, w_router, top, score="softmax", correction=None, n_groups=1, k
     return e, w
 
 
+def route_from_logits(logits_f32, top, score="softmax", correction=None, n_groups=1, keep_groups=1, dtype=torch.bfloat16):
+    rows, E = logits_f32.shape
+    e = torch.empty((rows, top), dtype=torch.int32, device=logits_f32.device)
+    w = torch.empty((rows, top), dtype=torch.float32, device=logits_f32.device)
+    _chk(ffi.lib().pegainfer_route_from_logits(_p(logits_f32), _p(correction), _p(e), _p(w), E, n_groups, keep_groups, top, rows,
+                                               1 if score == "softmax" else 0, 0 if dtype == torch.bfloat16 else 1, _stream()),
+         "route_from_logits")
+    return e, w
+
+
 def route_combine_add(y_pairs, weight, add, out_dtype):
     rows, top = weight.shape
     d = y_pairs.shape[1]

@@ -130,6 +130,11 @@ def test_softmax_router(dtype, experts, top):
     assert torch.equal(e.cpu().long().sort(-1).values, idx.sort(-1).values)
     close(wt.cpu().sort(-1).values, val.sort(-1).values, "float32", tol32=1e-5)
     assert float(wt.sum(-1).max()) < 1.0 or top == experts                       # the scores are not renormalised
+    # the form the runtime uses: logits by a GEMM into fp32, then the selection alone
+    logits = B().linear(dev(h, dtype), dev(wr, dtype), out_dtype=torch.float32)
+    e2, w2 = B().route_from_logits(logits, top, dtype=DT[dtype])
+    assert torch.equal(e2.cpu().long().sort(-1).values, idx.sort(-1).values)
+    close(w2.cpu().sort(-1).values, val.sort(-1).values, "float32", tol32=1e-5)
 
 
 def run_delta(cfg_m, w, p, h, dtype, lens_plan, eps=1e-5):
