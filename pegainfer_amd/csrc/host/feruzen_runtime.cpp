@@ -1039,7 +1039,9 @@ struct Model {
     const MlpCfg& f = c.mlp;
     const int ff = f.glu.ff, P = T * f.top;
     int32_t *t_group = tiles, *t_row0 = tiles + max_tiles, *t_rows = tiles + 2 * max_tiles, *n_tiles = tiles + 3 * max_tiles;
-    {  // router logits in fp32 by a GEMM over the stored values, then softmax over all experts and the top choices per row
+    if (T > 8) {   // many rows: one workgroup per row does logits and selection
+      FZ_K(pegainfer_route_topk(xb, w.router, nullptr, route_e, route_w, D, f.experts, 1, 1, f.top, T, PEGAINFER_SCORE_SOFTMAX, dtype, S()));
+    } else {       // few rows (decoding): the few-rows GEMM streams the router with the whole chip into fp32 logits, then the selection
       pegainfer_gemm_desc r{};
       r.x = xb; r.w = w.router; r.y = route_logits;
       r.x_dtype = r.w_dtype = dtype; r.y_dtype = PEGAINFER_DTYPE_F32;
