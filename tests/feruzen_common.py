@@ -88,6 +88,17 @@ def config_real_heads():
     ])
 
 
+def config_only_delta():
+    """no attention anywhere (no cache part at all), seven layers deep: the depth-weighted sum runs over up to eight streams"""
+    return base(40, 33, 2, 3, [delta(2, 1, 8, 12, 2 + i % 3, dense(24, 1.5) if i % 2 else None) for i in range(7)])
+
+
+def config_only_parallel():
+    """no delta layer anywhere"""
+    return base(56, 45, 4, 2, [parallel(left(2, 1, 12, 20, 4), right(2, 10, 6, 4.0), 1.1, 0.9, moe(16, 1.0, 3, 3)),
+                               parallel(left(3, 3, 8, 8, 8, base=77.0), right(1, 16, 24, 20.0), 0.5, 2.0, dense(40, 3.0))])
+
+
 def config_tiny():
     return base(48, 50, 2, 2, [delta(2, 2, 8, 8, 2, dense(32, 1.5)),
                                parallel(left(2, 1, 8, 8, 8), right(2, 8, 8, 10.0), 1.0, 1.0, moe(16, 1.5, 4, 2, shared=(16, 1.5)))])
@@ -101,7 +112,7 @@ def random_weights(cfg, seed=0, gate_gain=6.0):
     """{name: float32 tensor holding bf16 values}.  gate_gain: size of the matrix memory's gate inputs; 6 drives them into
     the cap, which a bf16 run cannot follow: there the rounding of the gate inputs alone, summed over the log forget gates
     of a few dozen tokens, moves old entries against new ones by tens of percent (the restatement itself moves that much
-    when its gate inputs are rounded to bf16), so bf16 runs take weights_for(), with gates a quarter that size."""
+    when its gate inputs are rounded to bf16), so bf16 runs take weights_for(), with gates a quarter that size (the delta rule's decay input scales along)."""
     g = torch.Generator().manual_seed(seed)
     D, V, K = cfg["width"], cfg["vocab"], cfg["canon"]["taps"]
     w = {}
@@ -131,7 +142,7 @@ def random_weights(cfg, seed=0, gate_gain=6.0):
                 lin("%s.%s" % (q, n), rows, D, 2.0)
                 w["%s.%s.conv" % (q, n)] = bf16_round(0.5 * torch.randn(rows, m["conv"], generator=g))
             lin(q + ".b", m["heads"], D, 2.0)
-            lin(q + ".a", m["heads"], D, 2.0)
+            lin(q + ".a", m["heads"], D, gate_gain / 3.0)       # the decay's input: its rounding adds up over the tokens, too
             vec(q + ".A_log", m["heads"], -0.5, 0.7)
             vec(q + ".dt_bias", m["heads"], 0.0, 0.5)
             vec(q + ".norm", m["vdim"], 1.0, 0.2)

@@ -13,7 +13,7 @@ import feruzen_common as C
 
 pytestmark = pytest.mark.gpu
 
-CONFIGS = {"real": C.config_real_heads, "a": C.config_a, "b": C.config_b, "odd": C.config_odd, "wide": C.config_wide_heads, "tiny": C.config_tiny}
+CONFIGS = {"real": C.config_real_heads, "only_delta": C.config_only_delta, "only_parallel": C.config_only_parallel, "a": C.config_a, "b": C.config_b, "odd": C.config_odd, "wide": C.config_wide_heads, "tiny": C.config_tiny}
 
 
 def check(got, ref, dtype, what=""):
@@ -34,8 +34,12 @@ def check(got, ref, dtype, what=""):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b", "odd", "wide", "tiny", "real"])
+@pytest.mark.parametrize("name", ["a", "b", "odd", "wide", "tiny", "real", "only_delta", "only_parallel"])
 def test_whole_prompt_every_position_and_every_layer(name, dtype):
+    if name == "only_delta" and dtype == "bfloat16":
+        # seven tiny delta layers, each normed on its OUTPUT: the plain restatement itself moves by 0.16 (median over rows,
+        # 0.5 at the 90 % quantile) when only its GEMM inputs and outputs are rounded to bf16 - nothing to hold a bf16 run to
+        pytest.skip("ill-conditioned in bf16: the restatement with bf16-rounded products is as far from itself")
     cfg = CONFIGS[name]()
     w = C.weights_for(cfg, 11, dtype)
     toks = C.tokens_for(cfg, 70, 1)
@@ -61,8 +65,12 @@ def test_whole_prompt_every_position_and_every_layer(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "odd", "wide", "real"])
+@pytest.mark.parametrize("name", ["a", "odd", "wide", "real", "only_delta", "only_parallel"])
 def test_prefill_then_token_by_token(name, dtype):
+    if name == "only_delta" and dtype == "bfloat16":
+        # seven tiny delta layers, each normed on its OUTPUT: the plain restatement itself moves by 0.16 (median over rows,
+        # 0.5 at the 90 % quantile) when only its GEMM inputs and outputs are rounded to bf16 - nothing to hold a bf16 run to
+        pytest.skip("ill-conditioned in bf16: the restatement with bf16-rounded products is as far from itself")
     cfg = CONFIGS[name]()
     w = C.weights_for(cfg, 12, dtype)
     toks = C.tokens_for(cfg, 60, 2)
