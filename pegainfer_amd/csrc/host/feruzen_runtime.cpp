@@ -1039,7 +1039,8 @@ struct Model {
     const MlpCfg& f = c.mlp;
     const int ff = f.glu.ff, P = T * f.top;
     int32_t *t_group = tiles, *t_row0 = tiles + max_tiles, *t_rows = tiles + 2 * max_tiles, *n_tiles = tiles + 3 * max_tiles;
-    if (T > 8) {   // many rows: one workgroup per row does logits and selection
+    if (T > 8 || f.experts > 1024) {   // many rows (or more experts than the selection kernel's four rows hold in LDS): one
+                                       // workgroup per row does logits and selection
       FZ_K(pegainfer_route_topk(xb, w.router, nullptr, route_e, route_w, D, f.experts, 1, 1, f.top, T, PEGAINFER_SCORE_SOFTMAX, dtype, S()));
     } else {       // few rows (decoding): the few-rows GEMM streams the router with the whole chip into fp32 logits, then the selection
       pegainfer_gemm_desc r{};
